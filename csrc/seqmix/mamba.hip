@@ -1,0 +1,169 @@
+// Mamba-2 (state-space duality) layer pieces.
+//   conv : causal per-channel convolution over the x|B|C channels + bias + silu; the inputs
+//          before a portion's first token come from the sequence's saved tail (the last
+//          taps-1 raw inputs), or are zero at the start of a sequence.
+//   scan : per head an N x P fp32 state, S <- exp(-exp(A_log) dt) S + dt B x^T,
+//          y = S^T C + D x, y *= silu(z); dt = softplus(raw + bias).  One thread owns value
+//          column p of S in registers; B, C, x, z, dt of a chunk of tokens go through LDS.
+//          The block of head 0 also rolls the convolution tail forward.
+#include "common.h"
+using namespace sm;
+
+template <typename T>
+__global__ void mamba_conv_k(const T* __restrict__ zx, int ldz, int xoff,
+                             const float* __restrict__ cw, const float* __restrict__ cb,
+                             const float* __restrict__ tail, const int* __restrict__ ent,
+                             const int* __restrict__ row_ent, float* __restrict__ out, int R,
+                             int C, int K) {
+  int c = blockIdx.x * blockDim.x + threadIdx.x;
+  int r = blockIdx.y;
+  if (c >= C) return;
+  Entry en = load_entry(ent, row_ent[r]);
+  int t = r - en.row0;
+  float acc = cb[c];
+  for (int kk = 0; kk < K; kk++) {
+    int q = t - (K - 1) + kk;
+    float val = 0.0f;
+    if (q >= 0) val = ldf(zx, (size_t)(en.row0 + q) * ldz + xoff + c);
+    else if (en.start > 0) val = tail[((size_t)en.slot * (K - 1) + (K - 1 + q)) * C + c];
+    acc += cw[(size_t)c * K + kk] * val;
+  }
+  out[(size_t)r * C + c] = acc * sigmoidf_(acc);
+}
+
+template <typename T, int NP>
+__global__ void __launch_bounds__(256)
+mamba_scan_k(const float* __restrict__ conv, int C, const T* __restrict__ zx, int ldz, int xoff,
+             int dtoff, const float* __restrict__ dt_bias, const float* __restrict__ A_log,
+             const float* __restrict__ Dp, float* __restrict__ state, float* __restrict__ tail,
+             const int* __restrict__ ent, float* __restrict__ y, int H, int P, int N, int G,
+             int K, int CT) {
+  int e = blockIdx.x / H, h = blockIdx.x % H;
+  Entry en = load_entry(ent, e);
+  if (en.n <= 0) return;
+  extern __shared__ float smem[];
+  float* sB = smem;                // [CT][NP]
+  float* sC = sB + CT * NP;        // [CT][NP]
+  float* sx = sC + CT * NP;        // [CT][P]
+  float* sz = sx + CT * P;         // [CT][P]
+  float* sdt = sz + CT * P;        // [CT]
+  float* sdA = sdt + CT;           // [CT]
+  int inner = H * P;
+  int g = h / (H / G);
+  int p = threadIdx.x;
+  bool act = p < P;
+  float S[NP];
+  float* Sg = state + ((size_t)en.slot * H + h) * N * P;
+#pragma unroll
+  for (int n = 0; n < NP; n++) S[n] = (act && n < N && en.start > 0) ? Sg[(size_t)n * P + p] : 0.0f;
+  float A = -expf(A_log[h]), Dh = Dp[h], bias = dt_bias[h];
+  for (int t0 = 0; t0 < en.n; t0 += CT) {
+    int ct = min(CT, en.n - t0);
+    for (int idx = threadIdx.x; idx < ct * NP; idx += blockDim.x) {
+      int t = idx / NP, n = idx % NP;
+      size_t row = (size_t)(en.row0 + t0 + t);
+      float b = 0.f, c = 0.f;
+      if (n < N) {
+        b = conv[row * C + inner + g * N + n];
+        c = conv[row * C + inner + G * N + g * N + n];
+      }
+      sB[idx] = b; sC[idx] = c;
+    }
+    for (int idx = threadIdx.x; idx < ct * P; idx += blockDim.x) {
+      int t = idx / P, q = idx % P;
+      size_t row = (size_t)(en.row0 + t0 + t);
+      sx[idx] = conv[row * C + h * P + q];
+      sz[idx] = ldf(zx, row * ldz + h * P + q);
+    }
+    for (int t = threadIdx.x; t < ct; t += blockDim.x) {
+      size_t row = (size_t)(en.row0 + t0 + t);
+      float dt = softplusf_(ldf(zx, row * ldz + dtoff + h) + bias);
+      sdt[t] = dt;
+      sdA[t] = expf(A * dt);
+    }
+    __syncthreads();
+    if (act) {
+      for (int t = 0; t < ct; t++) {
+        float dA = sdA[t], xp = sx[t * P + p];
+        float dx = sdt[t] * xp;
+        float acc = 0.0f;
+#pragma unroll
+        for (int n = 0; n < NP; n++) {
+          S[n] = dA * S[n] + dx * sB[t * NP + n];
+          acc += S[n] * sC[t * NP + n];
+        }
+        acc += Dh * xp;
+        float z = sz[t * P + p];
+        y[(size_t)(en.row0 + t0 + t) * inner + h * P + p] = acc * (z * sigmoidf_(z));
+      }
+    }
+    __syncthreads();
+  }
+  if (act) {
+#pragma unroll
+    for (int n = 0; n < NP; n++)
+      if (n < N) Sg[(size_t)n * P + p] = S[n];
+  }
+  if (h == 0 && K > 1) {
+    // new tail = the last K-1 raw inputs of (old tail ++ this portion); slot j reads old
+    // slot j + n or a row of the portion, so ascending j never reads a slot already written
+    float* tl = tail + (size_t)en.slot * (K - 1) * C;
+    for (int c = threadIdx.x; c < C; c += blockDim.x) {
+      for (int j = 0; j < K - 1; j++) {
+        int q = en.n + j - (K - 1);
+        float val;
+        if (q >= 0) val = ldf(zx, (size_t)(en.row0 + q) * ldz + xoff + c);
+        else val = en.start > 0 ? tl[(size_t)(K - 1 + q) * C + c] : 0.0f;
+        tl[(size_t)j * C + c] = val;
+      }
+    }
+  }
+}
+
+template <typename T, int NP>
+static int launch_ms(const float* conv, int C, const void* zx, int ldz, int xoff, int dtoff,
+                     const float* dt_bias, const float* A_log, const float* Dp, float* state,
+                     float* tail, const int* ent, int E, float* y, int H, int P, int N, int G,
+                     int K, hipStream_t st) {
+  int threads = ((P + 63) / 64) * 64;
+  int per = 2 * NP + 2 * P + 2;
+  int CT = (48 * 1024) / (per * 4);
+  if (CT > 32) CT = 32;
+  if (CT < 1) CT = 1;
+  size_t shm = (size_t)CT * per * 4;
+  hipLaunchKernelGGL((mamba_scan_k<T, NP>), dim3(E * H), dim3(threads), shm, st, conv, C,
+                     (const T*)zx, ldz, xoff, dtoff, dt_bias, A_log, Dp, state, tail, ent, y, H,
+                     P, N, G, K, CT);
+  return (int)hipGetLastError();
+}
+
+extern "C" {
+
+int p2p_sm_mamba_conv(const void* zx, int ldz, int xoff, const float* cw, const float* cb,
+                      const float* tail, const int* ent, const int* row_ent, float* out, int R,
+                      int C, int K, int f32, hipStream_t st) {
+  if (R <= 0) return 0;
+  dim3 g((C + 255) / 256, R), b(256);
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(mamba_conv_k<T>, g, b, 0, st, (const T*)zx, ldz, xoff, cw,
+                                         cb, tail, ent, row_ent, out, R, C, K));
+  return (int)hipGetLastError();
+}
+
+int p2p_sm_mamba_scan(const float* conv, int C, const void* zx, int ldz, int xoff, int dtoff,
+                      const float* dt_bias, const float* A_log, const float* Dp, float* state,
+                      float* tail, const int* ent, int E, float* y, int H, int P, int N, int G,
+                      int K, int f32, hipStream_t st) {
+  if (E <= 0) return 0;
+  if (N < 1 || N > 256 || P < 1 || P > 256 || G < 1 || H % G) return (int)hipErrorInvalidValue;
+#define MS(NPV)                                                                               \
+  SM_DISPATCH_T(f32, return (launch_ms<T, NPV>(conv, C, zx, ldz, xoff, dtoff, dt_bias, A_log, \
+                                               Dp, state, tail, ent, E, y, H, P, N, G, K, st)))
+  if (N <= 32) MS(32);
+  else if (N <= 64) MS(64);
+  else if (N <= 128) MS(128);
+  else MS(256);
+#undef MS
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,105 @@
+// Embedding with learned positions, RMS norms over fp32 or activation-typed rows (whole
+// row or equal parts, optional scatter of the rows), and the post-sublayer
+// norm + layer scale + residual add on the fp32 residual stream.
+#include "common.h"
+using namespace sm;
+
+template <typename T>
+__global__ void embed_pos_k(const T* __restrict__ embed, const T* __restrict__ ptab,
+                            const int* __restrict__ ids, const int* __restrict__ pos,
+                            float* __restrict__ out, int W, int has_pos) {
+  int r = blockIdx.x;
+  size_t eo = (size_t)ids[r] * W, po = (size_t)pos[r] * W;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float v = ldf(embed, eo + i);
+    if (has_pos) v += ldf(ptab, po + i);
+    out[(size_t)r * W + i] = v;
+  }
+}
+
+// one block per (row, part): out = x / sqrt(mean(x^2) + eps) * w
+template <typename TI, typename TO>
+__global__ void rmsnorm_k(const TI* __restrict__ x, int ldx, const float* __restrict__ w,
+                          TO* __restrict__ out, int ldo, const int* __restrict__ in_rows,
+                          const int* __restrict__ out_rows, int n, int parts, float eps) {
+  __shared__ float red[16];
+  int r = blockIdx.x / parts, g = blockIdx.x % parts;
+  int np = n / parts;
+  int ri = in_rows ? in_rows[r] : r;
+  const TI* xr = x + (size_t)ri * ldx + (size_t)g * np;
+  float ss = 0.0f;
+  for (int i = threadIdx.x; i < np; i += blockDim.x) {
+    float v = ldf(xr, i);
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  int ro = out_rows ? out_rows[r] : r;
+  if (ro < 0) return;
+  float rs = 1.0f / sqrtf(ss / (float)np + eps);
+  TO* o = out + (size_t)ro * ldo + (size_t)g * np;
+  for (int i = threadIdx.x; i < np; i += blockDim.x) {
+    float v = ldf(xr, i) * rs;
+    if (w) v *= w[g * np + i];
+    stf(o, i, v);
+  }
+}
+
+// x += y / sqrt(mean(y^2) + eps) * w * ls   (x fp32 residual)
+template <typename T>
+__global__ void norm_scale_add_k(float* __restrict__ x, const T* __restrict__ y, int ldy,
+                                 const float* __restrict__ w, const float* __restrict__ ls,
+                                 int n, float eps) {
+  __shared__ float red[16];
+  int r = blockIdx.x;
+  const T* yr = y + (size_t)r * ldy;
+  float ss = 0.0f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    float v = ldf(yr, i);
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  float rs = 1.0f / sqrtf(ss / (float)n + eps);
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    float v = ldf(yr, i) * rs * w[i];
+    if (ls) v *= ls[i];
+    x[(size_t)r * n + i] += v;
+  }
+}
+
+extern "C" {
+
+int p2p_sm_embed_pos(const void* embed, const void* ptab, const int* ids, const int* pos,
+                     float* out, int R, int W, int f32, hipStream_t st) {
+  if (R <= 0) return 0;
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(embed_pos_k<T>, dim3(R), dim3(256), 0, st,
+                                         (const T*)embed, (const T*)ptab, ids, pos, out, W,
+                                         ptab != nullptr));
+  return (int)hipGetLastError();
+}
+
+int p2p_sm_rmsnorm(const void* x, int ldx, int in_f32, const float* w, void* out, int ldo,
+                   int out_f32, const int* in_rows, const int* out_rows, int R, int n, int parts,
+                   float eps, hipStream_t st) {
+  if (R <= 0) return 0;
+  if (parts <= 0 || n % parts) return (int)hipErrorInvalidValue;
+  dim3 g(R * parts), b(256);
+#define RN(TI, TO)                                                                          \
+  hipLaunchKernelGGL((rmsnorm_k<TI, TO>), g, b, 0, st, (const TI*)x, ldx, w, (TO*)out, ldo, \
+                     in_rows, out_rows, n, parts, eps)
+  if (in_f32 && out_f32) RN(float, float);
+  else if (in_f32) RN(float, bf16);
+  else if (out_f32) RN(bf16, float);
+  else RN(bf16, bf16);
+#undef RN
+  return (int)hipGetLastError();
+}
+
+int p2p_sm_norm_scale_add(float* x, const void* y, int ldy, const float* w, const float* ls,
+                          int R, int n, float eps, int f32, hipStream_t st) {
+  if (R <= 0) return 0;
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(norm_scale_add_k<T>, dim3(R), dim3(256), 0, st, x,
+                                         (const T*)y, ldy, w, ls, n, eps));
+  return (int)hipGetLastError();
+}
+
+}  // extern "C"

@@ -1,0 +1,61 @@
+// Pointwise pieces between the matrix products: tanh in place, sigmoid output gates with
+// arbitrary input strides, and the clamped gated feed-forward activation
+//   g = min(gate, limit), u = clamp(up, -limit, limit), y = g * sigmoid(1.702 g) * (u + 1).
+#include "common.h"
+using namespace sm;
+
+template <typename T>
+__global__ void tanh_k(T* x, int ld, int n, int R) {
+  int c = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y;
+  if (c < n) stf(x, (size_t)r * ld + c, tanhf(ldf(x, (size_t)r * ld + c)));
+}
+
+// out[r, h * V + v] = o[h * soh + r * sor + v] * sigmoid(g[r * ldg + h * V + v])
+template <typename T>
+__global__ void sigmoid_gate_k(const T* __restrict__ o, long soh, long sor, const T* __restrict__ g,
+                               int ldg, T* __restrict__ out, int ldo, int H, int V) {
+  int c = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y;
+  if (c >= H * V) return;
+  int h = c / V, v = c % V;
+  float x = ldf(o, (size_t)h * soh + (size_t)r * sor + v);
+  stf(out, (size_t)r * ldo + c, x * sigmoidf_(ldf(g, (size_t)r * ldg + c)));
+}
+
+template <typename T>
+__global__ void ff_act_k(const T* __restrict__ gu, int ld, T* __restrict__ out, int ldo, int F,
+                         float limit, float alpha) {
+  int c = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y;
+  if (c >= F) return;
+  float g = fminf(ldf(gu, (size_t)r * ld + c), limit);
+  float u = fminf(fmaxf(ldf(gu, (size_t)r * ld + F + c), -limit), limit);
+  stf(out, (size_t)r * ldo + c, g * sigmoidf_(alpha * g) * (u + 1.0f));
+}
+
+extern "C" {
+
+int p2p_sm_tanh(void* x, int ld, int n, int R, int f32, hipStream_t st) {
+  if (R <= 0 || n <= 0) return 0;
+  dim3 g((n + 255) / 256, R), b(256);
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(tanh_k<T>, g, b, 0, st, (T*)x, ld, n, R));
+  return (int)hipGetLastError();
+}
+
+int p2p_sm_sigmoid_gate(const void* o, long soh, long sor, const void* gt, int ldg, void* out,
+                        int ldo, int R, int H, int V, int f32, hipStream_t st) {
+  if (R <= 0) return 0;
+  dim3 g((H * V + 255) / 256, R), b(256);
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(sigmoid_gate_k<T>, g, b, 0, st, (const T*)o, soh, sor,
+                                         (const T*)gt, ldg, (T*)out, ldo, H, V));
+  return (int)hipGetLastError();
+}
+
+int p2p_sm_ff_act(const void* gu, int ld, void* out, int ldo, int R, int F, float limit,
+                  float alpha, int f32, hipStream_t st) {
+  if (R <= 0) return 0;
+  dim3 g((F + 255) / 256, R), b(256);
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(ff_act_k<T>, g, b, 0, st, (const T*)gu, ld, (T*)out, ldo,
+                                         F, limit, alpha));
+  return (int)hipGetLastError();
+}
+
+}  // extern "C"

@@ -6,7 +6,7 @@ package (``p2p_llm_chat_go_amd/_lib``) so that they travel with the repo
 snapshot to the GPU box.  Targets are rebuilt only when a source or header is
 newer than the artefact.
 
-Usage:  python -m p2p_llm_chat_go_amd._build [--force] [--jobs N] [--only kernels|net|...]
+Usage:  python -m p2p_llm_chat_go_amd._build [--force] [--jobs N] [--only kernels|seqmix|native|experimental]
 """
 from __future__ import annotations
 
@@ -90,6 +90,39 @@ def _headers(d):
 
 
 EXPERIMENTAL_LIB = os.path.join(LIBDIR, "libp2p_experimental.so")
+# sequence-mixer kernels (recurrent state layers, latent attention, learned positions):
+# a library of their own, so a model that needs only these compiles only these
+SEQMIX_LIB = os.path.join(LIBDIR, "libp2p_seqmix.so")
+
+
+def seqmix_sources():
+    d = os.path.join(CSRC, "seqmix")
+    return sorted(glob.glob(os.path.join(d, "*.hip"))), sorted(glob.glob(os.path.join(d, "*.h")))
+
+
+def build_seqmix(force=False, jobs=8):
+    """Compile csrc/seqmix/*.hip for gfx950 into ``libp2p_seqmix.so`` (C ABI, ctypes)."""
+    srcs, hdrs = seqmix_sources()
+    odir = os.path.join(BUILDDIR, "seqmix")
+    os.makedirs(odir, exist_ok=True)
+    os.makedirs(LIBDIR, exist_ok=True)
+    flags = ["--offload-arch=%s" % ARCH, "-O3", "-fPIC", "-std=c++17", "-Xclang",
+             "-target-feature", "-Xclang", "-packed-fp32-ops", "-I", os.path.join(CSRC, "seqmix")]
+    objs, todo = [], []
+    for s in srcs:
+        o = os.path.join(odir, os.path.basename(s) + ".o")
+        objs.append(o)
+        if force or _stale(o, [s] + hdrs):
+            todo.append((s, o))
+    with cf.ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
+        for f in [ex.submit(_run, [HIPCC] + flags + ["-c", s, "-o", o]) for s, o in todo]:
+            f.result()
+    if force or todo or _stale(SEQMIX_LIB, objs):
+        tmp = SEQMIX_LIB + ".tmp.%d" % os.getpid()
+        _run([HIPCC, "-shared", "-fPIC", "--offload-arch=%s" % ARCH] + objs + ["-o", tmp])
+        os.replace(tmp, SEQMIX_LIB)
+    _write_stamp(SEQMIX_LIB, srcs, hdrs)
+    return SEQMIX_LIB
 
 
 # Kernels whose k loop streams through inline-asm loads (csrc/kernels/wide_gemm.hip): the
@@ -294,6 +327,8 @@ def build(force=False, jobs=8, only=None, experimental=None):
         # on by default: the experimental library's tests run on the GPU box, so the binary
         # they load must be built from HEAD like the rest (P2P_BUILD_EXPERIMENTAL=0 skips it)
         experimental = os.environ.get("P2P_BUILD_EXPERIMENTAL", "1") == "1"
+    if only in (None, "seqmix") and (shutil.which(HIPCC) or os.path.exists(HIPCC)):
+        outs.append(build_seqmix(force, jobs))
     if only in (None, "kernels", "experimental"):
         if shutil.which(HIPCC) or os.path.exists(HIPCC):
             if only != "experimental":
@@ -311,7 +346,7 @@ def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--force", action="store_true")
     ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
-    ap.add_argument("--only", choices=["kernels", "native", "experimental"], default=None)
+    ap.add_argument("--only", choices=["kernels", "native", "experimental", "seqmix"], default=None)
     ap.add_argument("--sanitize", choices=sorted(SANITIZERS), default=None,
                     help="build only the sanitizer variant of the daemons into bin/<kind>/")
     a = ap.parse_args(argv)
