@@ -39,6 +39,8 @@ PREFILL_CTX = int(os.environ.get("ENGINE_PREFILL_GRAPH_CTX", "4096"))
 
 
 def native_loop_ok(engine: Engine) -> bool:
+    if not isinstance(engine, Engine):  # other engine classes (hybrid models): Python loop
+        return False
     return (engine.device.type == "cuda" and engine.use_graph and engine.model.tp == 1
             and engine.prefill_graphs_enabled
             and os.environ.get("ENGINE_NATIVE_LOOP", "1") != "0")

@@ -97,6 +97,7 @@ class EngineServer:
         # the scheduler owns page allocation for served requests
         self._lock = threading.Condition()
         self._reqs = {}      # id -> dict(prompt, params, future, t_submit, t_admit, t_first)
+        self._page0 = {}     # id -> first page of an admitted request (names its sequence)
         self._pending = []   # (prompt_ids, params, future, t_submit) waiting to enter the scheduler
         self._cancels = set()  # futures whose requests should stop
         self._stop = False
@@ -328,7 +329,7 @@ class EngineServer:
                         r["future"].set_exception(e)
                     self.sched.cancel(rid)
                 for rid in self.sched.take_finished():
-                    self.sched.release(rid)  # scheduler entries + KV pages
+                    self._release(rid)  # scheduler entries + KV pages
                 self._reqs.clear()
                 self.errors += 1
                 if self.fatal(e):  # a TP peer is gone: this replica cannot serve again
@@ -358,6 +359,8 @@ class EngineServer:
         if plan.prefill:
             prompts = [self._reqs[i]["prompt"] for i in plan.prefill]
             pages = [list(self.sched.get(i).pages) for i in plan.prefill]
+            for i, pg in zip(plan.prefill, pages):
+                self._page0[i] = pg[0]
             ride = [i for i in plan.decode if self.sched.get(i).state == 1] if self.mixed else []
             # riders: every running sequence (within the chunk budget), or only the rows left
             # in the prefill's last 64-row GEMM tile
@@ -458,5 +461,14 @@ class EngineServer:
                     "eval_count": len(toks), "eval_duration": now - t_first,
                     "total_duration": now - r["t_submit"],
                     "ttft_ns": t_first - r["t_submit"]})
-            self.sched.release(rid)
+            self._release(rid)
         return done
+
+    def _release(self, rid):
+        """Give a finished request's pages back (and, for engines that keep per-sequence
+        state beside the pages, tell the engine first: its state slot is free again)."""
+        page0 = self._page0.pop(rid, None)
+        rel = getattr(self.engine, "release_sequence", None)
+        if rel is not None and page0 is not None:
+            rel([page0])
+        self.sched.release(rid)

@@ -94,8 +94,29 @@ ALIASES = {"llama3.1": "llama3.1-8b", "llama3.1:8b": "llama3.1-8b", "llama3.1:70
            "mixtral": "mixtral-8x7b", "mixtral:8x7b": "mixtral-8x7b", "tiny": "tiny-llama"}
 
 
-def get_config(name: str) -> ModelConfig:
+def _hybrid_presets() -> dict:
+    """Hybrid (recurrent + latent attention) presets, built on first use."""
+    from .hybrid import HybridConfig
+
+    gd = {"type": "general_delta", "mixer": {"heads": 4, "dim": 32}, "mlp": None}
+    mb = {"type": "mamba2", "mixer": {"heads": 8, "vdim": 32, "state": 32, "groups": 2, "conv": 4,
+                                      "norm_groups": 2}, "mlp": None}
+    la = {"type": "latent_attention",
+          "mixer": {"heads": 4, "dim": 32, "vdim": 32, "kv_rank": 64, "mask": {"size": 128},
+                    "scale": 32 ** -0.5},
+          "mlp": {"kind": "dense", "ff": 512, "limit": 7.0}}
+    return {"tiny-regesun": HybridConfig.from_dict(
+        {"architecture": "Regesun", "width": 256, "vocab": 512, "max_positions": 4096,
+         "norm": {"eps": 1e-5}, "layers": [gd, mb, la, mb, gd, la], "eos_token_id": [2]},
+        name="tiny-regesun")}
+
+
+def get_config(name: str):
     key = ALIASES.get(name, name)
+    if key not in PRESETS and key.endswith("regesun"):
+        hp = _hybrid_presets()
+        if key in hp:
+            return hp[key]
     if key not in PRESETS:
         raise KeyError("unknown model %r (known: %s)" % (name, ", ".join(sorted(PRESETS))))
     return PRESETS[key]

@@ -82,6 +82,18 @@ class HybridConfig:
                    max_pos=int(c["max_positions"]), bos_id=int(c.get("bos_token_id", 1)),
                    eos_ids=eos)
 
+    def resolve(self, shapes: dict) -> "HybridConfig":
+        """Fill the sizes that a config leaves to the checkpoint's tensor shapes (the rank of
+        the generalized delta rule's decay projection).  shapes: tensor name -> shape."""
+        layers = []
+        for i, L in enumerate(self.layers):
+            mx = dict(L.mixer)
+            k = "l%d.mix.w1" % i
+            if L.kind == "general_delta" and "decay_rank" not in mx and k in shapes:
+                mx["decay_rank"] = int(tuple(shapes[k])[0])
+            layers.append(LayerSpec(L.kind, mx, L.mlp))
+        return dataclasses.replace(self, layers=tuple(layers))
+
     def to_dict(self) -> dict:
         return {"architecture": "Regesun", "width": self.width, "vocab": self.vocab,
                 "max_positions": self.max_pos, "norm": {"eps": self.eps},
@@ -339,6 +351,7 @@ class HybridWeights:
     fp32.  ``dtype`` is torch.bfloat16 (serving) or torch.float32 (exact)."""
 
     def __init__(self, cfg: HybridConfig, sd, device, dtype=torch.bfloat16):
+        cfg = cfg.resolve({k: v.shape for k, v in sd.items()})
         self.cfg, self.dtype = cfg, dtype
         dev = self.device = torch.device(device)
         want = tensor_shapes(cfg)
@@ -402,7 +415,8 @@ def load_dir(path: str, device="cuda", dtype=torch.bfloat16):
     with open(os.path.join(path, "config.json")) as f:
         cfg = HybridConfig.from_dict(json.load(f), name=os.path.basename(os.path.normpath(path)))
     sd = load_file(os.path.join(path, "model.safetensors"))
-    return cfg, HybridWeights(cfg, sd, device, dtype)
+    w = HybridWeights(cfg, sd, device, dtype)
+    return w.cfg, w
 
 
 # ---------------------------------------------------------------------------- model

@@ -8,9 +8,11 @@ MYNAMEIS, HTTP_ADDR, DIRECTORY_URL, BOOTSTRAP_ADDRS -- plus opt-in extras
 STRICT_SENDER, UI_FILE) and the engine knobs:
 
   ENGINE          1 (default) / 0: attach the in-process engine
-  ENGINE_MODEL    preset name (default: llama3.1-8b on a GPU, tiny-llama on CPU)
+  ENGINE_MODEL    preset name (default: llama3.1-8b on a GPU, tiny-llama on CPU;
+                  tiny-regesun: a small hybrid recurrent / latent-attention model)
   ENGINE_DEVICE   cuda:N / cpu (default: cuda:0 if available)
-  ENGINE_CHECKPOINT  HF checkpoint dir (safetensors + config.json); default random-init
+  ENGINE_CHECKPOINT  checkpoint dir (safetensors + config.json: HF Llama / Mixtral, or a
+                  hybrid design named by its "architecture" key); default random-init
   ENGINE_MAX_BATCH   concurrent sequences (default 16)
   ENGINE_MAX_TOKENS  default num_predict (default 128)
   ENGINE_WARMUP   1 (default on GPUs): autotune GEMMs + capture decode graphs at start
@@ -49,27 +51,27 @@ def build_engine_server(model: str | None = None, device: str | None = None):
         return cluster.from_env(device)
     import torch
 
-    from ..engine import Engine
     from ..engine.native_loop import make_server
     from ..engine.tokenizer import get_tokenizer
+    from ..models import registry
     from ..models.config import get_config
-    from ..models.weights import (EngineWeights, config_from_hf, load_safetensors_dir)
 
     dev = device or os.environ.get("ENGINE_DEVICE") or ("cuda:0" if torch.cuda.is_available()
                                                         else "cpu")
     ckpt = os.environ.get("ENGINE_CHECKPOINT", "")
     max_batch = int(os.environ.get("ENGINE_MAX_BATCH", "16"))
     if ckpt:
-        cfg = config_from_hf(ckpt)
-        weights = EngineWeights.from_state_dict(load_safetensors_dir(ckpt, dev), cfg, dev)
+        # the checkpoint's config.json picks the model class (models.registry)
+        cfg, weights = registry.load_checkpoint(ckpt, dev)
     else:
         name = model or os.environ.get("ENGINE_MODEL") or (
             "llama3.1-8b" if str(dev).startswith("cuda") else "tiny-llama")
         cfg = get_config(name)
         weights = None
     kv_pages = None if str(dev).startswith("cuda") else 256
-    eng = Engine(cfg, weights=weights, device=dev, kv_pages=kv_pages, max_batch=max_batch)
-    if str(dev).startswith("cuda") and os.environ.get("ENGINE_WARMUP", "1") != "0":
+    eng = registry.make_engine(cfg, weights, dev, kv_pages=kv_pages, max_batch=max_batch)
+    if (hasattr(eng, "warmup") and str(dev).startswith("cuda")
+            and os.environ.get("ENGINE_WARMUP", "1") != "0"):
         # autotuned GEMM launch codes + decode graphs of the common batch buckets, before
         # the first request (ENGINE_WARMUP=0 skips: faster start, untuned first replies)
         eng.warmup(tuple(b for b in (1, 2, 4, 8, 16) if b <= max_batch), ctx=256)
