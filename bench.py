@@ -66,6 +66,14 @@ def parse(argv=None):
                     help="index into SAMPLE_MESSAGES for peer 0 (default: the median-length one)")
     ap.add_argument("--device", choices=("cuda", "cpu"), default="cuda",
                     help="cpu: gloo + the CPU engine (plumbing tests with tiny models)")
+    ap.add_argument("--hybrid", action="store_true",
+                    help="instead of the headline workload: prefill / decode throughput of "
+                         "Regesun hybrid models beside a dense Llama of equal size "
+                         "(bench/hybrid_bench.py; 1 GPU)")
+    ap.add_argument("--hybrid-sizes", default="1024,2048", help="model widths for --hybrid")
+    ap.add_argument("--hybrid-prompt", type=int, default=2048)
+    ap.add_argument("--hybrid-batch", type=int, default=8)
+    ap.add_argument("--hybrid-ctx", type=int, default=512)
     ap.add_argument("--layers", type=int, default=None,
                     help="override n_layers (tests only; a reduced model is not a valid bench)")
     return ap.parse_args(argv)
@@ -99,6 +107,11 @@ def launch(a, argv) -> int:
 def main(argv=None):
     argv = sys.argv[1:] if argv is None else argv
     a = parse(argv)
+    if a.hybrid:
+        sys.path.insert(0, os.path.join(ROOT, "bench"))
+        import hybrid_bench
+
+        return hybrid_bench.run(a)
     if "WORLD_SIZE" not in os.environ and a.gpus > 1:
         sys.exit(launch(a, argv))
     run(a)

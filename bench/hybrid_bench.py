@@ -1,0 +1,119 @@
+"""Prefill and decode throughput of hybrid (Regesun) models at layer sizes that resemble real
+models, beside a dense Llama of the same width, depth and parameter count on the same engine
+entry point (``generate``).  Random weights, random tokens.
+
+    python bench.py --hybrid [--hybrid-sizes 1024,2048] [--steps K] [--warmup W]
+
+One JSON line per (size, model): prefill tokens/s of one long prompt (``prompt`` tokens),
+decode tokens/s of ``batch`` sequences.  These lines are not the headline metric.
+"""
+from __future__ import annotations
+
+import json
+import time
+
+import torch
+
+
+def regesun_config(width: int):
+    """A Regesun stack at a given width: blocks of delta / mamba / mamba / attention+ff."""
+    from p2p_llm_chat_go_amd.models.hybrid import HybridConfig
+
+    hd = 64
+    gd = {"type": "general_delta", "mixer": {"heads": width // hd, "dim": hd}, "mlp": None}
+    mb = {"type": "mamba2", "mixer": {"heads": 2 * width // hd, "vdim": hd, "state": 128,
+                                      "groups": 8, "conv": 4, "norm_groups": 8}, "mlp": None}
+    la = {"type": "latent_attention",
+          "mixer": {"heads": width // 128, "dim": 128, "vdim": 128, "kv_rank": width // 4,
+                    "mask": {"size": 1024}, "scale": 128 ** -0.5},
+          "mlp": {"kind": "dense", "ff": 4 * width, "limit": 7.0}}
+    return HybridConfig.from_dict(
+        {"architecture": "Regesun", "width": width, "vocab": 32000, "max_positions": 8192,
+         "norm": {"eps": 1e-5}, "layers": [gd, mb, mb, la] * 4}, name="regesun-w%d" % width)
+
+
+def n_params(cfg) -> int:
+    from p2p_llm_chat_go_amd.models.hybrid import tensor_shapes
+
+    n = 0
+    for s in tensor_shapes(cfg.resolve({})).values():
+        k = 1
+        for d in s:
+            k *= d
+        n += k
+    return n
+
+
+def llama_like(width: int, layers: int, params: int):
+    """Dense Llama of the same width and depth whose ffn size makes the parameter count match."""
+    from p2p_llm_chat_go_amd.models.config import ModelConfig
+
+    nh = width // 128
+    nkv = max(1, nh // 4)
+    vocab = 32000
+    attn = width * (nh + 2 * nkv) * 128 + nh * 128 * width
+    per_layer = (params - 2 * vocab * width) / layers - attn
+    ffn = max(256, int(per_layer / (3 * width)) // 256 * 256)
+    return ModelConfig("llama-w%d" % width, hidden=width, n_layers=layers, n_heads=nh,
+                       n_kv_heads=nkv, ffn=ffn, vocab=vocab, max_pos=8192, rope_theta=10000.0,
+                       rope_llama3=None, bos_id=1, eos_ids=(2,))
+
+
+def measure(eng, vocab, prompt, batch, ctx, new_tokens, steps, warmup, dev):
+    g = torch.Generator().manual_seed(0)
+    long_p = [torch.randint(3, vocab, (prompt,), generator=g).tolist()]
+    many = [torch.randint(3, vocab, (ctx,), generator=g).tolist() for _ in range(batch)]
+    out = {}
+    for name, prompts, new in (("prefill", long_p, 2), ("decode", many, new_tokens)):
+        for _ in range(warmup):
+            eng.generate(prompts, new, stop_on_eos=False)
+        torch.cuda.synchronize(dev)
+        pre = dec = 0.0
+        for _ in range(steps):
+            r = eng.generate(prompts, new, stop_on_eos=False)[0]
+            pre += r.ttft_ns * 1e-9
+            dec += r.eval_duration_ns * 1e-9
+        torch.cuda.synchronize(dev)
+        if name == "prefill":
+            out["prefill_tok_s"] = round(steps * prompt / pre, 1)
+            out["prefill_ms"] = round(1e3 * pre / steps, 3)
+        else:
+            out["decode_tok_s"] = round(steps * batch * (new - 1) / dec, 1)
+            out["decode_ms_per_step"] = round(1e3 * dec / (steps * (new - 1)), 3)
+    return out
+
+
+def run(a):
+    from p2p_llm_chat_go_amd.engine import Engine
+    from p2p_llm_chat_go_amd.models import registry
+
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    prompt, batch, ctx, new = a.hybrid_prompt, a.hybrid_batch, a.hybrid_ctx, a.new_tokens
+    pages = max(prompt // 64 + 4, batch * ((ctx + new) // 64 + 2)) + 8
+    for width in [int(w) for w in a.hybrid_sizes.split(",")]:
+        hcfg = regesun_config(width)
+        params = n_params(hcfg)
+        lcfg = llama_like(width, hcfg.n_layers, params)
+        for cfg in (hcfg, lcfg):
+            hybrid = cfg is hcfg
+            if hybrid:
+                eng = registry.make_engine(cfg, None, dev, kv_pages=pages, max_batch=batch,
+                                           max_prefill_tokens=prompt, seed=1)
+            else:
+                eng = Engine(cfg, device=dev, seed=1, kv_pages=pages, max_prefill_tokens=prompt,
+                             max_batch=batch)
+                eng.warmup((batch,), ctx=ctx + new)
+            t0 = time.perf_counter()
+            m = measure(eng, cfg.vocab, prompt, batch, ctx, new, a.steps, a.warmup, dev)
+            line = {"metric": "hybrid-vs-dense throughput", "model": cfg.name,
+                    "params_m": round((params if hybrid else cfg.n_params()) / 1e6, 1),
+                    "width": width, "layers": cfg.n_layers, "dtype": "bf16",
+                    "prompt_tokens": prompt, "decode_batch": batch, "decode_ctx": ctx,
+                    "new_tokens": new, "steps": a.steps, "warmup": a.warmup,
+                    "data": "random tokens; random-init weights",
+                    "bench_s": round(time.perf_counter() - t0, 1)}
+            line.update(m)
+            print(json.dumps(line), flush=True)
+            del eng
+            torch.cuda.empty_cache()

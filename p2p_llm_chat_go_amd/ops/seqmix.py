@@ -369,13 +369,9 @@ def mamba_scan(conv, zx, xoff: int, dtoff: int, dt_bias, A_log, Dp, state, tail,
 
 
 # ------------------------------------------------------------------ latent attention
-LATENT_MAX_PAIRS = 32 * 256     # heads x latent size one block accumulates
-LATENT_MAX_LDS = 64 * 1024
-
-
 def latent_attn_ok(H: int, rank: int) -> bool:
-    lds = (H * rank + 32 * (rank + 1) + H * 32 + 3 * H) * 4
-    return H <= 256 and H * rank <= LATENT_MAX_PAIRS and lds <= LATENT_MAX_LDS
+    """One head's query, a tile of 4 keys and the accumulators must fit a block."""
+    return rank <= 32 * 256 and (rank + 4 * (rank + 1) + 4 + 3) * 4 <= 64 * 1024
 
 
 def latent_attn(qa, cache, block_tables, row_ent, pos, sink, scale: float, win: int, out,
