@@ -5,7 +5,7 @@
 //   scan : per head an N x P fp32 state, S <- exp(-exp(A_log) dt) S + dt B x^T,
 //          y = S^T C + D x, y *= silu(z); dt = softplus(raw + bias).  One thread owns value
 //          column p of S in registers; B, C, x, z, dt of a chunk of tokens go through LDS.
-//          The block of head 0 also rolls the convolution tail forward.
+//   tail : rolls the convolution tail forward after the scan.
 #include "common.h"
 using namespace sm;
 
@@ -104,19 +104,25 @@ mamba_scan_k(const float* __restrict__ conv, int C, const T* __restrict__ zx, in
     for (int n = 0; n < NP; n++)
       if (n < N) Sg[(size_t)n * P + p] = S[n];
   }
-  if (h == 0 && K > 1) {
-    // new tail = the last K-1 raw inputs of (old tail ++ this portion); slot j reads old
-    // slot j + n or a row of the portion, so ascending j never reads a slot already written
-    float* tl = tail + (size_t)en.slot * (K - 1) * C;
-    for (int c = threadIdx.x; c < C; c += blockDim.x) {
-      for (int j = 0; j < K - 1; j++) {
-        int q = en.n + j - (K - 1);
-        float val;
-        if (q >= 0) val = ldf(zx, (size_t)(en.row0 + q) * ldz + xoff + c);
-        else val = en.start > 0 ? tl[(size_t)(K - 1 + q) * C + c] : 0.0f;
-        tl[(size_t)j * C + c] = val;
-      }
-    }
+}
+
+// new tail = the last K-1 raw inputs of (old tail ++ this portion): one thread per (entry,
+// channel); slot j reads old slot j + n or a row of the portion, so ascending j never reads
+// a slot it has already written
+template <typename T>
+__global__ void mamba_tail_k(const T* __restrict__ zx, int ldz, int xoff, float* __restrict__ tail,
+                             const int* __restrict__ ent, int C, int K) {
+  int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  Entry en = load_entry(ent, blockIdx.y);
+  if (en.n <= 0) return;
+  float* tl = tail + (size_t)en.slot * (K - 1) * C;
+  for (int j = 0; j < K - 1; j++) {
+    int q = en.n + j - (K - 1);
+    float val;
+    if (q >= 0) val = ldf(zx, (size_t)(en.row0 + q) * ldz + xoff + c);
+    else val = en.start > 0 ? tl[(size_t)(K - 1 + q) * C + c] : 0.0f;
+    tl[(size_t)j * C + c] = val;
   }
 }
 
@@ -164,6 +170,15 @@ int p2p_sm_mamba_scan(const float* conv, int C, const void* zx, int ldz, int xof
   else MS(256);
 #undef MS
   return 0;
+}
+
+int p2p_sm_mamba_tail(const void* zx, int ldz, int xoff, float* tail, const int* ent, int E, int C,
+                      int K, int f32, hipStream_t st) {
+  if (E <= 0 || K <= 1) return 0;
+  dim3 g((C + 255) / 256, E), b(256);
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(mamba_tail_k<T>, g, b, 0, st, (const T*)zx, ldz, xoff, tail,
+                                        ent, C, K));
+  return (int)hipGetLastError();
 }
 
 }  // extern "C"

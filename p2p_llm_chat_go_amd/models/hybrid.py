@@ -148,6 +148,15 @@ class StepBatch:
         self.ent = cut[4].view(-1, 4)
         self.out_rows = cut[5][:self.n_out]
         self.block_tables = cut[6].view(len(entries), maxp)
+        self._units = {}
+
+    def units(self, rows_per_wave: int):
+        """Row groups for the matrix-core attention kernel (``ops.seqmix.make_units``)."""
+        u = self._units.get(rows_per_wave)
+        if u is None:
+            u = self._units[rows_per_wave] = sm.make_units(self.ent_host, rows_per_wave).to(
+                self.ids.device)
+        return u
 
 
 # ---------------------------------------------------------------------------- mixers
@@ -289,8 +298,9 @@ class LatentAttention(Mixer):
         sm.rmsnorm(proj[:, H * D:H * D + r], self.cnorm, self.eps, pool, out_rows=b.cache_rows)
         qa = torch.bmm(proj[:, :H * D].view(b.R, H, D).transpose(0, 1), self.uk)   # [H, R, rank]
         ol = torch.empty_like(qa)
+        units = b.units(sm.latent_rows_per_wave(H)) if sm.latent_mfma_ok(qa, pool) else None
         sm.latent_attn(qa, pool, b.block_tables, b.row_ent, b.pos, self.sink, self.scale, self.win,
-                       ol, PAGE)
+                       ol, PAGE, units=units)
         o = torch.bmm(ol, self.uvt)                                                # [H, R, V]
         gated = torch.empty(b.R, H * V, device=h.device, dtype=h.dtype)
         sm.sigmoid_gate(o, proj[:, H * D + r:], gated, H, V)

@@ -42,9 +42,14 @@ _SIGS = {
     "p2p_sm_mamba_scan": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p,
                           c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
                           c_int, c_int, c_int, c_int, c_void_p],
+    "p2p_sm_mamba_tail": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                          c_void_p],
     "p2p_sm_latent_attn": [c_void_p, c_long, c_long, c_void_p, c_void_p, c_int, c_void_p,
                            c_void_p, c_void_p, c_float, c_int, c_void_p, c_long, c_long, c_int,
                            c_int, c_int, c_int, c_int, c_void_p],
+    "p2p_sm_latent_attn_mfma": [c_void_p, c_long, c_long, c_void_p, c_void_p, c_int, c_void_p,
+                                c_void_p, c_void_p, c_int, c_void_p, c_float, c_int, c_void_p,
+                                c_long, c_long, c_int, c_int, c_int, c_void_p],
     "p2p_sm_tanh": [c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "p2p_sm_sigmoid_gate": [c_void_p, c_long, c_long, c_void_p, c_int, c_void_p, c_int, c_int,
                             c_int, c_int, c_int, c_void_p],
@@ -365,6 +370,8 @@ def mamba_scan(conv, zx, xoff: int, dtoff: int, dt_bias, A_log, Dp, state, tail,
                                  state.data_ptr(), tail.data_ptr(), ent.data_ptr(), E,
                                  y.data_ptr(), H, P, N, G, Km1 + 1, _f32(zx), _st(zx)),
          "mamba_scan")
+    _chk(lib().p2p_sm_mamba_tail(zx.data_ptr(), zx.stride(0), xoff, tail.data_ptr(),
+                                 ent.data_ptr(), E, C, Km1 + 1, _f32(zx), _st(zx)), "mamba_tail")
     return y
 
 
@@ -374,15 +381,43 @@ def latent_attn_ok(H: int, rank: int) -> bool:
     return rank <= 32 * 256 and (rank + 4 * (rank + 1) + 4 + 3) * 4 <= 64 * 1024
 
 
+def latent_rows_per_wave(H: int) -> int:
+    """Rows of one sequence portion that a wavefront of the matrix-core kernel takes: its 16
+    (row, head) pairs are RW rows x HS head slots, HS the power of two >= min(H, 16)."""
+    hs = 1
+    while hs < H and hs < 16:
+        hs *= 2
+    return 16 // hs
+
+
+def make_units(ent_host: list, rows_per_wave: int) -> torch.Tensor:
+    """int32 [U, 2] (first row, rows): the entries' rows cut into groups of at most
+    ``rows_per_wave`` consecutive rows; a group never spans two entries."""
+    u = [(r, min(rows_per_wave, row0 + n - r)) for row0, n, _s, _sl in ent_host
+         for r in range(row0, row0 + n, rows_per_wave)]
+    return torch.tensor(u, dtype=torch.int32).view(-1, 2)
+
+
+def latent_mfma_ok(qa, cache) -> bool:
+    """The matrix-core kernel serves bf16 activations with a latent size that is a multiple
+    of 8 up to 512 and 16-byte aligned rows; everything else (and float32) runs the fp32
+    kernel.  P2P_LATENT_MFMA=0 switches it off."""
+    rank = qa.shape[2]
+    return (qa.is_cuda and qa.dtype == torch.bfloat16 and rank % 8 == 0 and 8 <= rank <= 512
+            and qa.stride(0) % 8 == 0 and qa.stride(1) % 8 == 0 and qa.data_ptr() % 16 == 0
+            and cache.data_ptr() % 16 == 0 and os.environ.get("P2P_LATENT_MFMA", "1") != "0")
+
+
 def latent_attn(qa, cache, block_tables, row_ent, pos, sink, scale: float, win: int, out,
-                page: int):
+                page: int, units=None):
     """Windowed attention over cached latents with a softmax sink.
 
     qa [H, R, rank] (any strides, last = 1): the queries already carried into latent space
     (W_uk^T q per head); cache [tokens, rank] one layer's latent pool, token t of a sequence
     at block_tables[e, t // page] * page + t % page.  out [H, R, rank] = sum_j p_j c_j with
     p = softmax over {sink_h} U {scale * qa . c_j : 0 <= pos - j < win}, the sink term having
-    no value."""
+    no value.  units: ``make_units(entries, latent_rows_per_wave(H))`` on the device; with
+    it, bf16 inputs run on the matrix cores (``latent_mfma_ok``)."""
     H, R, rank = qa.shape
     if not qa.is_cuda:
         bt = block_tables.long()
@@ -404,6 +439,16 @@ def latent_attn(qa, cache, block_tables, row_ent, pos, sink, scale: float, win: 
     assert block_tables.dtype == torch.int32 and block_tables.is_contiguous()
     assert row_ent.dtype == torch.int32 and pos.dtype == torch.int32
     _vec(sink, H, "sink")
+    if units is not None and latent_mfma_ok(qa, cache):
+        assert units.dtype == torch.int32 and units.is_contiguous() and units.shape[1] == 2
+        _chk(lib().p2p_sm_latent_attn_mfma(qa.data_ptr(), qa.stride(0), qa.stride(1),
+                                           cache.data_ptr(), block_tables.data_ptr(),
+                                           block_tables.shape[1], row_ent.data_ptr(),
+                                           pos.data_ptr(), units.data_ptr(), units.shape[0],
+                                           sink.data_ptr(), scale, win, out.data_ptr(),
+                                           out.stride(0), out.stride(1), H, rank, page, _st(qa)),
+             "latent_attn_mfma")
+        return out
     if not latent_attn_ok(H, rank):
         raise ValueError("latent_attn: %d heads x latent %d exceed the kernel's tile" % (H, rank))
     _chk(lib().p2p_sm_latent_attn(qa.data_ptr(), qa.stride(0), qa.stride(1), cache.data_ptr(),

@@ -120,7 +120,7 @@ def test_mamba(dt, H, P, N, G, K):
 
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,rank,win", [(6, 120, 36), (3, 40, 7), (5, 96, 200)])
+@pytest.mark.parametrize("H,rank,win", [(6, 120, 36), (3, 40, 7), (5, 96, 200), (16, 512, 33), (20, 64, 64), (1, 8, 3)])
 def test_latent_attn(dt, H, rank, win):
     g = torch.Generator().manual_seed(4)
     page, npages = 64, 12
@@ -136,3 +136,11 @@ def test_latent_attn(dt, H, rank, win):
     b = sm.latent_attn(qa.to(DEV), cache.to(DEV), bt.to(DEV), row_ent.to(DEV), pos.to(DEV), sink.to(DEV), 0.2,
                        win, torch.empty(H, R, rank, dtype=dt, device=DEV), page)
     torch.testing.assert_close(b.cpu().float(), a.float(), **_tol(dt))
+    if dt == torch.bfloat16:
+        # the matrix-core kernel: queries as a contiguous [H, R, rank] tensor, row groups per wave
+        qc = qa.contiguous().to(DEV)
+        assert sm.latent_mfma_ok(qc, cache.to(DEV))
+        units = sm.make_units([(0, 40, 100, 0), (40, 1, 70, 1)], sm.latent_rows_per_wave(H)).to(DEV)
+        c = sm.latent_attn(qc, cache.to(DEV), bt.to(DEV), row_ent.to(DEV), pos.to(DEV), sink.to(DEV), 0.2,
+                           win, torch.empty(H, R, rank, dtype=dt, device=DEV), page, units=units)
+        torch.testing.assert_close(c.cpu().float(), a.float(), **_tol(dt))
