@@ -17,8 +17,14 @@ gdelta_scan_k(const T* __restrict__ r, const T* __restrict__ k, const T* __restr
               const T* __restrict__ lo, int ldlo, const float* __restrict__ w0,
               const float* __restrict__ ab, const float* __restrict__ normw,
               float* __restrict__ state, const int* __restrict__ ent, T* __restrict__ out,
-              int ldo, int H, int D, float eps, int CT) {
+              int ldo, int H, int D, float eps, int CT, int mode, float* __restrict__ state2) {
+  // mode 0: a portion from its slot's state (or zero at position 0), state written back.
+  // mode 1: a chunk alone, no outputs: blockIdx.y = 0 runs it from a zero state and leaves the
+  //         end state in state[slot]; blockIdx.y = 1 runs only the state transition on the
+  //         identity (no k v^T term) and leaves the chunk's transition matrix in state2[slot].
+  // mode 2: a chunk from state[slot], outputs only.
   int e = blockIdx.x / H, h = blockIdx.x % H;
+  const bool trans = mode == 1 && blockIdx.y == 1;
   Entry en = load_entry(ent, e);
   if (en.n <= 0) return;
   extern __shared__ float smem[];
@@ -31,9 +37,13 @@ gdelta_scan_k(const T* __restrict__ r, const T* __restrict__ k, const T* __restr
   int j = threadIdx.x;
   bool act = j < D;
   float S[DKP];
-  float* Sg = state + ((size_t)en.slot * H + h) * D * D;
+  float* Sg = (trans ? state2 : state) + ((size_t)en.slot * H + h) * D * D;
+  const bool from_state = mode == 2 || (mode == 0 && en.start > 0);
 #pragma unroll
-  for (int i = 0; i < DKP; i++) S[i] = (act && i < D && en.start > 0) ? Sg[(size_t)i * D + j] : 0.0f;
+  for (int i = 0; i < DKP; i++) {
+    float v0 = trans ? (i == j ? 1.0f : 0.0f) : 0.0f;
+    S[i] = (act && i < D && from_state) ? Sg[(size_t)i * D + j] : v0;
+  }
   int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   for (int t0 = 0; t0 < en.n; t0 += CT) {
     int ct = min(CT, en.n - t0);
@@ -64,7 +74,7 @@ gdelta_scan_k(const T* __restrict__ r, const T* __restrict__ k, const T* __restr
         }
         float rs = 1.0f / sqrtf(kk + 1e-6f);
         float dot = d * rs;            // u^T S (column j)
-        float vj = sv[t * DKP + j];
+        float vj = trans ? 0.0f : sv[t * DKP + j];
         float o = 0.0f;
 #pragma unroll
         for (int i = 0; i < DKP; i++) {
@@ -77,6 +87,7 @@ gdelta_scan_k(const T* __restrict__ r, const T* __restrict__ k, const T* __restr
       }
     }
     __syncthreads();
+    if (mode != 1)
     for (int t = wave; t < ct; t += nw) {
       float ss = 0.0f;
       for (int i = lane; i < D; i += 64) ss += so[t * DKP + i] * so[t * DKP + i];
@@ -93,10 +104,60 @@ gdelta_scan_k(const T* __restrict__ r, const T* __restrict__ k, const T* __restr
     // written again only after the next first barrier, which every wave reaches after its
     // share of this chunk's outputs
   }
-  if (act) {
+  if (act && mode != 2) {
 #pragma unroll
     for (int i = 0; i < DKP; i++)
       if (i < D) Sg[(size_t)i * D + j] = S[i];
+  }
+}
+
+// Chains the chunks of each portion: init_{c+1} = trans_c . init_c + local_c (D x D products
+// on the key index).  One block per (portion, head), one thread per value column.  `init`
+// receives init_c for every chunk, the portion's slot its final state.
+template <int DKP>
+__global__ void __launch_bounds__(256)
+gdelta_combine_k(const float* __restrict__ local, const float* __restrict__ trans,
+                 float* __restrict__ init, float* __restrict__ state,
+                 const int* __restrict__ cent, int H, int D, int TI) {
+  extern __shared__ float sP[];   // [TI][D] rows of the transition matrix
+  int e = blockIdx.x / H, h = blockIdx.x % H;
+  int c0 = cent[4 * e], nc = cent[4 * e + 1], start = cent[4 * e + 2], slot = cent[4 * e + 3];
+  int j = threadIdx.x;
+  bool act = j < D;
+  size_t DD = (size_t)D * D;
+  float* sg = state + ((size_t)slot * H + h) * DD;
+  float cur[DKP];
+#pragma unroll
+  for (int k = 0; k < DKP; k++) cur[k] = (act && k < D && start > 0) ? sg[(size_t)k * D + j] : 0.0f;
+  for (int c = c0; c < c0 + nc; c++) {
+    size_t off = ((size_t)c * H + h) * DD;
+    if (act) {
+#pragma unroll
+      for (int k = 0; k < DKP; k++)
+        if (k < D) init[off + (size_t)k * D + j] = cur[k];
+    }
+    float* dst = (c + 1 < c0 + nc) ? init + ((size_t)(c + 1) * H + h) * DD : sg;
+    for (int i0 = 0; i0 < D; i0 += TI) {
+      int ti = min(TI, D - i0);
+      __syncthreads();
+      for (int idx = threadIdx.x; idx < ti * D; idx += blockDim.x)
+        sP[idx] = trans[off + (size_t)i0 * D + idx];
+      __syncthreads();
+      if (act) {
+        for (int i = 0; i < ti; i++) {
+          float a = local[off + (size_t)(i0 + i) * D + j];
+#pragma unroll
+          for (int k = 0; k < DKP; k++)
+            if (k < D) a += sP[i * D + k] * cur[k];
+          dst[(size_t)(i0 + i) * D + j] = a;
+        }
+      }
+    }
+    if (act) {
+#pragma unroll
+      for (int k = 0; k < DKP; k++)
+        if (k < D) cur[k] = dst[(size_t)k * D + j];
+    }
   }
 }
 
@@ -104,28 +165,31 @@ template <typename T, int DKP>
 static int launch_gd(const void* r, const void* k, const void* v, const void* g, const void* a,
                      int ld, const void* lo, int ldlo, const float* w0, const float* ab,
                      const float* normw, float* state, const int* ent, int E, void* out, int ldo,
-                     int H, int D, float eps, hipStream_t st) {
+                     int H, int D, float eps, int mode, float* state2, hipStream_t st) {
   int threads = ((D + 63) / 64) * 64;
   int CT = (48 * 1024) / (6 * DKP * 4);
   if (CT > 32) CT = 32;
   if (CT < 1) CT = 1;
   size_t shm = (size_t)6 * CT * DKP * 4;
-  hipLaunchKernelGGL((gdelta_scan_k<T, DKP>), dim3(E * H), dim3(threads), shm, st, (const T*)r,
-                     (const T*)k, (const T*)v, (const T*)g, (const T*)a, ld, (const T*)lo, ldlo,
-                     w0, ab, normw, state, ent, (T*)out, ldo, H, D, eps, CT);
+  hipLaunchKernelGGL((gdelta_scan_k<T, DKP>), dim3(E * H, mode == 1 ? 2 : 1), dim3(threads), shm,
+                     st, (const T*)r, (const T*)k, (const T*)v, (const T*)g, (const T*)a, ld,
+                     (const T*)lo, ldlo, w0, ab, normw, state, ent, (T*)out, ldo, H, D, eps, CT,
+                     mode, state2);
   return (int)hipGetLastError();
 }
 
-extern "C" int p2p_sm_gdelta_scan(const void* r, const void* k, const void* v, const void* g,
-                                  const void* a, int ld, const void* lo, int ldlo,
-                                  const float* w0, const float* ab, const float* normw,
-                                  float* state, const int* ent, int E, void* out, int ldo, int H,
-                                  int D, float eps, int f32, hipStream_t st) {
+extern "C" {
+
+int p2p_sm_gdelta_scan_mode(const void* r, const void* k, const void* v, const void* g,
+                            const void* a, int ld, const void* lo, int ldlo, const float* w0,
+                            const float* ab, const float* normw, float* state, const int* ent,
+                            int E, void* out, int ldo, int H, int D, float eps, int mode,
+                            float* state2, int f32, hipStream_t st) {
   if (E <= 0) return 0;
   if (D < 1 || D > 256) return (int)hipErrorInvalidValue;
 #define GD(P)                                                                                   \
   SM_DISPATCH_T(f32, return (launch_gd<T, P>(r, k, v, g, a, ld, lo, ldlo, w0, ab, normw, state, \
-                                             ent, E, out, ldo, H, D, eps, st)))
+                                             ent, E, out, ldo, H, D, eps, mode, state2, st)))
   if (D <= 32) GD(32);
   else if (D <= 64) GD(64);
   else if (D <= 128) GD(128);
@@ -133,3 +197,46 @@ extern "C" int p2p_sm_gdelta_scan(const void* r, const void* k, const void* v, c
 #undef GD
   return 0;
 }
+
+int p2p_sm_gdelta_scan(const void* r, const void* k, const void* v, const void* g, const void* a,
+                       int ld, const void* lo, int ldlo, const float* w0, const float* ab,
+                       const float* normw, float* state, const int* ent, int E, void* out,
+                       int ldo, int H, int D, float eps, int f32, hipStream_t st) {
+  return p2p_sm_gdelta_scan_mode(r, k, v, g, a, ld, lo, ldlo, w0, ab, normw, state, ent, E, out,
+                                 ldo, H, D, eps, 0, nullptr, f32, st);
+}
+
+// Long portions in chunks that run side by side: every chunk's local end state and transition
+// matrix, a chain over each portion's chunks, then every chunk again from its true initial
+// state.  vent: the chunks as entries (row0, n, 1, chunk index); tmp: 3 fp32 buffers of
+// [chunks, H, D, D] (local, transition, init); cent: per portion (first chunk, chunks, first
+// position, slot).
+int p2p_sm_gdelta_scan_chunked(const void* r, const void* k, const void* v, const void* g,
+                               const void* a, int ld, const void* lo, int ldlo, const float* w0,
+                               const float* ab, const float* normw, float* state, float* tmp,
+                               const int* vent, int NV, const int* cent, int E, void* out,
+                               int ldo, int H, int D, float eps, int f32, hipStream_t st) {
+  if (E <= 0 || NV <= 0) return 0;
+  size_t sz = (size_t)NV * H * D * D;
+  float *loc = tmp, *trn = tmp + sz, *ini = tmp + 2 * sz;
+  int err = p2p_sm_gdelta_scan_mode(r, k, v, g, a, ld, lo, ldlo, w0, ab, normw, loc, vent, NV, out,
+                                    ldo, H, D, eps, 1, trn, f32, st);
+  if (err) return err;
+  int threads = ((D + 63) / 64) * 64;
+  int TI = (32 * 1024) / (D * 4);
+  if (TI > D) TI = D;
+  if (TI < 1) TI = 1;
+  size_t shm = (size_t)TI * D * 4;
+#define GC(P) hipLaunchKernelGGL((gdelta_combine_k<P>), dim3(E * H), dim3(threads), shm, st, loc, trn, ini, state, cent, H, D, TI)
+  if (D <= 32) GC(32);
+  else if (D <= 64) GC(64);
+  else if (D <= 128) GC(128);
+  else GC(256);
+#undef GC
+  err = (int)hipGetLastError();
+  if (err) return err;
+  return p2p_sm_gdelta_scan_mode(r, k, v, g, a, ld, lo, ldlo, w0, ab, normw, ini, vent, NV, out,
+                                 ldo, H, D, eps, 2, nullptr, f32, st);
+}
+
+}  // extern "C"

@@ -37,7 +37,11 @@ mamba_scan_k(const float* __restrict__ conv, int C, const T* __restrict__ zx, in
              int dtoff, const float* __restrict__ dt_bias, const float* __restrict__ A_log,
              const float* __restrict__ Dp, float* __restrict__ state, float* __restrict__ tail,
              const int* __restrict__ ent, float* __restrict__ y, int H, int P, int N, int G,
-             int K, int CT) {
+             int K, int CT, int mode, float* __restrict__ decay_out) {
+  // mode 0: a portion from its slot's state (or zero at position 0), state written back.
+  // mode 1: a chunk from a zero state: no outputs; the end state goes to `state[slot]` and
+  //         the product of the chunk's decays to decay_out[entry, head].
+  // mode 2: a chunk from `state[slot]`, outputs only.
   int e = blockIdx.x / H, h = blockIdx.x % H;
   Entry en = load_entry(ent, e);
   if (en.n <= 0) return;
@@ -54,9 +58,11 @@ mamba_scan_k(const float* __restrict__ conv, int C, const T* __restrict__ zx, in
   bool act = p < P;
   float S[NP];
   float* Sg = state + ((size_t)en.slot * H + h) * N * P;
+  const bool from_state = mode == 2 || (mode == 0 && en.start > 0);
 #pragma unroll
-  for (int n = 0; n < NP; n++) S[n] = (act && n < N && en.start > 0) ? Sg[(size_t)n * P + p] : 0.0f;
+  for (int n = 0; n < NP; n++) S[n] = (act && n < N && from_state) ? Sg[(size_t)n * P + p] : 0.0f;
   float A = -expf(A_log[h]), Dh = Dp[h], bias = dt_bias[h];
+  float dtsum = 0.0f;
   for (int t0 = 0; t0 < en.n; t0 += CT) {
     int ct = min(CT, en.n - t0);
     for (int idx = threadIdx.x; idx < ct * NP; idx += blockDim.x) {
@@ -85,6 +91,7 @@ mamba_scan_k(const float* __restrict__ conv, int C, const T* __restrict__ zx, in
     if (act) {
       for (int t = 0; t < ct; t++) {
         float dA = sdA[t], xp = sx[t * P + p];
+        dtsum += sdt[t];
         float dx = sdt[t] * xp;
         float acc = 0.0f;
 #pragma unroll
@@ -94,16 +101,38 @@ mamba_scan_k(const float* __restrict__ conv, int C, const T* __restrict__ zx, in
         }
         acc += Dh * xp;
         float z = sz[t * P + p];
-        y[(size_t)(en.row0 + t0 + t) * inner + h * P + p] = acc * (z * sigmoidf_(z));
+        if (mode != 1) y[(size_t)(en.row0 + t0 + t) * inner + h * P + p] = acc * (z * sigmoidf_(z));
       }
     }
     __syncthreads();
   }
-  if (act) {
+  if (act && mode != 2) {
 #pragma unroll
     for (int n = 0; n < NP; n++)
       if (n < N) Sg[(size_t)n * P + p] = S[n];
   }
+  if (mode == 1 && p == 0) decay_out[(size_t)e * H + h] = expf(A * dtsum);
+}
+
+// Chains the chunks of each portion: chunk c starts from init_c, init_{c+1} = decay_c * init_c
+// + local_c.  `tmp` holds local_c on entry and init_c on exit; the portion's final state goes
+// to its slot.  cent: per portion (first chunk, chunks, first position, slot).
+__global__ void mamba_combine_k(float* __restrict__ tmp, const float* __restrict__ decay,
+                                float* __restrict__ state, const int* __restrict__ cent, int H,
+                                int NPsz) {
+  int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= NPsz) return;
+  int h = blockIdx.y, e = blockIdx.z;
+  int c0 = cent[4 * e], nc = cent[4 * e + 1], start = cent[4 * e + 2], slot = cent[4 * e + 3];
+  float* sg = state + ((size_t)slot * H + h) * NPsz + idx;
+  float cur = start > 0 ? *sg : 0.0f;
+  for (int c = c0; c < c0 + nc; c++) {
+    float* t = tmp + ((size_t)c * H + h) * NPsz + idx;
+    float loc = *t;
+    *t = cur;
+    cur = decay[(size_t)c * H + h] * cur + loc;
+  }
+  *sg = cur;
 }
 
 // new tail = the last K-1 raw inputs of (old tail ++ this portion): one thread per (entry,
@@ -130,7 +159,7 @@ template <typename T, int NP>
 static int launch_ms(const float* conv, int C, const void* zx, int ldz, int xoff, int dtoff,
                      const float* dt_bias, const float* A_log, const float* Dp, float* state,
                      float* tail, const int* ent, int E, float* y, int H, int P, int N, int G,
-                     int K, hipStream_t st) {
+                     int K, int mode, float* decay_out, hipStream_t st) {
   int threads = ((P + 63) / 64) * 64;
   int per = 2 * NP + 2 * P + 2;
   int CT = (48 * 1024) / (per * 4);
@@ -139,7 +168,7 @@ static int launch_ms(const float* conv, int C, const void* zx, int ldz, int xoff
   size_t shm = (size_t)CT * per * 4;
   hipLaunchKernelGGL((mamba_scan_k<T, NP>), dim3(E * H), dim3(threads), shm, st, conv, C,
                      (const T*)zx, ldz, xoff, dtoff, dt_bias, A_log, Dp, state, tail, ent, y, H,
-                     P, N, G, K, CT);
+                     P, N, G, K, CT, mode, decay_out);
   return (int)hipGetLastError();
 }
 
@@ -155,21 +184,51 @@ int p2p_sm_mamba_conv(const void* zx, int ldz, int xoff, const float* cw, const 
   return (int)hipGetLastError();
 }
 
-int p2p_sm_mamba_scan(const float* conv, int C, const void* zx, int ldz, int xoff, int dtoff,
-                      const float* dt_bias, const float* A_log, const float* Dp, float* state,
-                      float* tail, const int* ent, int E, float* y, int H, int P, int N, int G,
-                      int K, int f32, hipStream_t st) {
+int p2p_sm_mamba_scan_mode(const float* conv, int C, const void* zx, int ldz, int xoff,
+                           int dtoff, const float* dt_bias, const float* A_log, const float* Dp,
+                           float* state, float* tail, const int* ent, int E, float* y, int H,
+                           int P, int N, int G, int K, int mode, float* decay_out, int f32,
+                           hipStream_t st) {
   if (E <= 0) return 0;
   if (N < 1 || N > 256 || P < 1 || P > 256 || G < 1 || H % G) return (int)hipErrorInvalidValue;
 #define MS(NPV)                                                                               \
   SM_DISPATCH_T(f32, return (launch_ms<T, NPV>(conv, C, zx, ldz, xoff, dtoff, dt_bias, A_log, \
-                                               Dp, state, tail, ent, E, y, H, P, N, G, K, st)))
+                                               Dp, state, tail, ent, E, y, H, P, N, G, K, mode, \
+                                               decay_out, st)))
   if (N <= 32) MS(32);
   else if (N <= 64) MS(64);
   else if (N <= 128) MS(128);
   else MS(256);
 #undef MS
   return 0;
+}
+
+int p2p_sm_mamba_scan(const float* conv, int C, const void* zx, int ldz, int xoff, int dtoff,
+                      const float* dt_bias, const float* A_log, const float* Dp, float* state,
+                      float* tail, const int* ent, int E, float* y, int H, int P, int N, int G,
+                      int K, int f32, hipStream_t st) {  return p2p_sm_mamba_scan_mode(conv, C, zx, ldz, xoff, dtoff, dt_bias, A_log, Dp, state, tail,
+                                ent, E, y, H, P, N, G, K, 0, nullptr, f32, st);
+}
+
+// Long portions in chunks that run side by side: local states of every chunk from zero, a
+// chain over each portion's chunks, then every chunk again from its true initial state.
+// vent: the chunks as entries (row0, n, 1, chunk index); tmp fp32 [chunks, H, N, P];
+// decay fp32 [chunks, H]; cent: see mamba_combine_k.
+int p2p_sm_mamba_scan_chunked(const float* conv, int C, const void* zx, int ldz, int xoff,
+                              int dtoff, const float* dt_bias, const float* A_log,
+                              const float* Dp, float* state, float* tmp, float* decay,
+                              const int* vent, int NV, const int* cent, int E, float* y, int H,
+                              int P, int N, int G, int f32, hipStream_t st) {
+  if (E <= 0 || NV <= 0) return 0;
+  int err = p2p_sm_mamba_scan_mode(conv, C, zx, ldz, xoff, dtoff, dt_bias, A_log, Dp, tmp,
+                                   nullptr, vent, NV, y, H, P, N, G, 1, 1, decay, f32, st);
+  if (err) return err;
+  dim3 g((N * P + 255) / 256, H, E);
+  hipLaunchKernelGGL(mamba_combine_k, g, dim3(256), 0, st, tmp, decay, state, cent, H, N * P);
+  err = (int)hipGetLastError();
+  if (err) return err;
+  return p2p_sm_mamba_scan_mode(conv, C, zx, ldz, xoff, dtoff, dt_bias, A_log, Dp, tmp, nullptr,
+                                vent, NV, y, H, P, N, G, 1, 2, nullptr, f32, st);
 }
 
 int p2p_sm_mamba_tail(const void* zx, int ldz, int xoff, float* tail, const int* ent, int E, int C,

@@ -37,6 +37,14 @@ _SIGS = {
     "p2p_sm_gdelta_scan": [c_void_p] * 5 + [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                                             c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
                                             c_int, c_float, c_int, c_void_p],
+    "p2p_sm_gdelta_scan_chunked": [c_void_p] * 5 + [c_int, c_void_p, c_int, c_void_p, c_void_p,
+                                                    c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                                    c_void_p, c_int, c_void_p, c_int, c_int, c_int,
+                                                    c_float, c_int, c_void_p],
+    "p2p_sm_mamba_scan_chunked": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p,
+                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                  c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int,
+                                  c_int, c_void_p],
     "p2p_sm_mamba_conv": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "p2p_sm_mamba_scan": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p,
@@ -247,6 +255,30 @@ def ff_act(gu, out, limit: float, alpha: float = 1.702):
     return out
 
 
+# ------------------------------------------------------------------ recurrences in chunks
+# A portion of at least 2 * SCAN_CHUNK tokens is scanned in chunks of SCAN_CHUNK tokens that
+# run side by side (local pass, chain over the chunks, output pass); shorter steps -- decode,
+# small portions -- walk their tokens in one pass.  Both recurrences are linear in the state,
+# so the chunked form computes the same sums in another order (fp32 throughout).
+SCAN_CHUNK = int(os.environ.get("P2P_SCAN_CHUNK", "64"))
+
+
+def scan_chunks(ent_host: list, chunk: int):
+    """(chunks as entries [(row0, n, 1, chunk index)], per entry (first chunk, chunks, first
+    position, slot)) as int32 tensors."""
+    vent, cent = [], []
+    for row0, n, start, slot in ent_host:
+        c0 = len(vent)
+        for r in range(row0, row0 + n, chunk):
+            vent.append((r, min(chunk, row0 + n - r), 1, len(vent)))
+        cent.append((c0, len(vent) - c0, start, slot))
+    return torch.tensor(vent, dtype=torch.int32), torch.tensor(cent, dtype=torch.int32)
+
+
+def _chunked(ent_host) -> bool:
+    return SCAN_CHUNK > 0 and max(e[1] for e in ent_host) >= 2 * SCAN_CHUNK
+
+
 # ------------------------------------------------------------------ generalized delta rule
 GD_DECAY_SCALE = math.exp(-0.5)
 
@@ -288,6 +320,15 @@ def gdelta_scan(r, k, v, g, a, lo, w0, ab, normw, state, ent, ent_host, out, H: 
     assert ent.dtype == torch.int32 and ent.is_contiguous() and ent.shape[1] == 4
     if D > 256:
         raise ValueError("gdelta_scan: head size %d > 256" % D)
+    if _chunked(ent_host):
+        vent, cent = (t_.to(r.device) for t_ in scan_chunks(ent_host, SCAN_CHUNK))
+        tmp = torch.empty(3, vent.shape[0], H, D, D, device=r.device, dtype=torch.float32)
+        _chk(lib().p2p_sm_gdelta_scan_chunked(
+            r.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), a.data_ptr(), ld,
+            lo.data_ptr(), lo.stride(0), w0.data_ptr(), ab.data_ptr(), normw.data_ptr(),
+            state.data_ptr(), tmp.data_ptr(), vent.data_ptr(), vent.shape[0], cent.data_ptr(), E,
+            out.data_ptr(), out.stride(0), H, D, eps, _f32(r), _st(r)), "gdelta_scan_chunked")
+        return out
     _chk(lib().p2p_sm_gdelta_scan(r.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(),
                                   a.data_ptr(), ld, lo.data_ptr(), lo.stride(0), w0.data_ptr(),
                                   ab.data_ptr(), normw.data_ptr(), state.data_ptr(),
@@ -365,11 +406,22 @@ def mamba_scan(conv, zx, xoff: int, dtoff: int, dt_bias, A_log, Dp, state, tail,
     if N > 256 or P > 256:
         raise ValueError("mamba_scan: state %d / value %d sizes above 256" % (N, P))
     E = ent.shape[0]
-    _chk(lib().p2p_sm_mamba_scan(conv.data_ptr(), C, zx.data_ptr(), zx.stride(0), xoff, dtoff,
-                                 dt_bias.data_ptr(), A_log.data_ptr(), Dp.data_ptr(),
-                                 state.data_ptr(), tail.data_ptr(), ent.data_ptr(), E,
-                                 y.data_ptr(), H, P, N, G, Km1 + 1, _f32(zx), _st(zx)),
-         "mamba_scan")
+    if _chunked(ent_host):
+        vent, cent = (t_.to(zx.device) for t_ in scan_chunks(ent_host, SCAN_CHUNK))
+        NV = vent.shape[0]
+        tmp = torch.empty(NV, H, N, P, device=zx.device, dtype=torch.float32)
+        decay = torch.empty(NV, H, device=zx.device, dtype=torch.float32)
+        _chk(lib().p2p_sm_mamba_scan_chunked(
+            conv.data_ptr(), C, zx.data_ptr(), zx.stride(0), xoff, dtoff, dt_bias.data_ptr(),
+            A_log.data_ptr(), Dp.data_ptr(), state.data_ptr(), tmp.data_ptr(), decay.data_ptr(),
+            vent.data_ptr(), NV, cent.data_ptr(), E, y.data_ptr(), H, P, N, G, _f32(zx),
+            _st(zx)), "mamba_scan_chunked")
+    else:
+        _chk(lib().p2p_sm_mamba_scan(conv.data_ptr(), C, zx.data_ptr(), zx.stride(0), xoff, dtoff,
+                                     dt_bias.data_ptr(), A_log.data_ptr(), Dp.data_ptr(),
+                                     state.data_ptr(), tail.data_ptr(), ent.data_ptr(), E,
+                                     y.data_ptr(), H, P, N, G, Km1 + 1, _f32(zx), _st(zx)),
+             "mamba_scan")
     _chk(lib().p2p_sm_mamba_tail(zx.data_ptr(), zx.stride(0), xoff, tail.data_ptr(),
                                  ent.data_ptr(), E, C, Km1 + 1, _f32(zx), _st(zx)), "mamba_tail")
     return y

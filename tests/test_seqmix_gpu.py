@@ -71,9 +71,17 @@ def test_pointwise(dt):
     torch.testing.assert_close(b.cpu().float(), a.float(), **_tol(dt))
 
 
+@pytest.fixture(params=[64, 8], ids=["onepass", "chunks8"])
+def scan_chunk(request, monkeypatch):
+    """Both forms of the recurrent scans: one pass over a portion, and chunks of 8 tokens
+    side by side (used for portions of 16 tokens and more)."""
+    monkeypatch.setattr(sm, "SCAN_CHUNK", request.param)
+    return request.param
+
+
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,D", [(2, 40), (3, 20), (1, 72)])
-def test_gdelta(dt, H, D):
+def test_gdelta(dt, H, D, scan_chunk):
     g = torch.Generator().manual_seed(2)
     n = H * D
     slots = 5
@@ -95,7 +103,7 @@ def test_gdelta(dt, H, D):
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,P,N,G,K", [(6, 40, 24, 3, 3), (4, 24, 16, 1, 4), (2, 72, 80, 2, 2)])
-def test_mamba(dt, H, P, N, G, K):
+def test_mamba(dt, H, P, N, G, K, scan_chunk):
     g = torch.Generator().manual_seed(3)
     inner, C = H * P, H * P + 2 * G * N
     slots = 4
