@@ -41,8 +41,11 @@ gdelta_scan_k(const T* __restrict__ r, const T* __restrict__ k, const T* __restr
   const bool from_state = mode == 2 || (mode == 0 && en.start > 0);
 #pragma unroll
   for (int i = 0; i < DKP; i++) {
+    // loads at clamped addresses, selected afterwards: the loads stay independent of the
+    // bounds tests and go out together
     float v0 = trans ? (i == j ? 1.0f : 0.0f) : 0.0f;
-    S[i] = (act && i < D && from_state) ? Sg[(size_t)i * D + j] : v0;
+    float v = from_state ? Sg[(size_t)min(i, D - 1) * D + min(j, D - 1)] : v0;
+    S[i] = (act && i < D) ? v : 0.0f;
   }
   int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   for (int t0 = 0; t0 < en.n; t0 += CT) {
@@ -119,16 +122,21 @@ __global__ void __launch_bounds__(256)
 gdelta_combine_k(const float* __restrict__ local, const float* __restrict__ trans,
                  float* __restrict__ init, float* __restrict__ state,
                  const int* __restrict__ cent, int H, int D, int TI) {
-  extern __shared__ float sP[];   // [TI][D] rows of the transition matrix
+  extern __shared__ float sP[];   // [TI (+3)][DS] rows of the transition matrix, zero padded
+  const int DS = (D + 3) & ~3;
   int e = blockIdx.x / H, h = blockIdx.x % H;
   int c0 = cent[4 * e], nc = cent[4 * e + 1], start = cent[4 * e + 2], slot = cent[4 * e + 3];
   int j = threadIdx.x;
   bool act = j < D;
+  int jc = min(j, D - 1);
   size_t DD = (size_t)D * D;
   float* sg = state + ((size_t)slot * H + h) * DD;
   float cur[DKP];
 #pragma unroll
-  for (int k = 0; k < DKP; k++) cur[k] = (act && k < D && start > 0) ? sg[(size_t)k * D + j] : 0.0f;
+  for (int k = 0; k < DKP; k++) {
+    float v = start > 0 ? sg[(size_t)min(k, D - 1) * D + jc] : 0.0f;
+    cur[k] = (act && k < D) ? v : 0.0f;
+  }
   for (int c = c0; c < c0 + nc; c++) {
     size_t off = ((size_t)c * H + h) * DD;
     if (act) {
@@ -140,23 +148,37 @@ gdelta_combine_k(const float* __restrict__ local, const float* __restrict__ tran
     for (int i0 = 0; i0 < D; i0 += TI) {
       int ti = min(TI, D - i0);
       __syncthreads();
-      for (int idx = threadIdx.x; idx < ti * D; idx += blockDim.x)
-        sP[idx] = trans[off + (size_t)i0 * D + idx];
+      for (int idx = threadIdx.x; idx < (ti + 3) * DS; idx += blockDim.x) {
+        int i = idx / DS, k = idx % DS;
+        sP[idx] = (i < ti && k < D) ? trans[off + (size_t)(i0 + i) * D + k] : 0.0f;
+      }
       __syncthreads();
       if (act) {
-        for (int i = 0; i < ti; i++) {
-          float a = local[off + (size_t)(i0 + i) * D + j];
+        for (int i = 0; i < ti; i += 4) {   // four rows at a time: independent sums
+          float a[4];
 #pragma unroll
-          for (int k = 0; k < DKP; k++)
-            if (k < D) a += sP[i * D + k] * cur[k];
-          dst[(size_t)(i0 + i) * D + j] = a;
+          for (int u = 0; u < 4; u++)
+            a[u] = local[off + (size_t)min(i0 + i + u, D - 1) * D + j];
+#pragma unroll
+          for (int k = 0; k < DKP; k += 4) {
+            if (k < DS) {
+#pragma unroll
+              for (int u = 0; u < 4; u++) {
+                const float4 p = *(const float4*)(sP + (i + u) * DS + k);
+                a[u] += p.x * cur[k] + p.y * cur[k + 1] + p.z * cur[k + 2] + p.w * cur[k + 3];
+              }
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < 4; u++)
+            if (i + u < ti) dst[(size_t)(i0 + i + u) * D + j] = a[u];
         }
       }
     }
-    if (act) {
 #pragma unroll
-      for (int k = 0; k < DKP; k++)
-        if (k < D) cur[k] = dst[(size_t)k * D + j];
+    for (int k = 0; k < DKP; k++) {
+      float v = dst[(size_t)min(k, D - 1) * D + jc];   // this thread's own column, just written
+      cur[k] = (act && k < D) ? v : 0.0f;
     }
   }
 }
@@ -223,10 +245,11 @@ int p2p_sm_gdelta_scan_chunked(const void* r, const void* k, const void* v, cons
                                     ldo, H, D, eps, 1, trn, f32, st);
   if (err) return err;
   int threads = ((D + 63) / 64) * 64;
-  int TI = (32 * 1024) / (D * 4);
+  int DS = (D + 3) & ~3;
+  int TI = ((32 * 1024) / (DS * 4)) & ~3;
   if (TI > D) TI = D;
-  if (TI < 1) TI = 1;
-  size_t shm = (size_t)TI * D * 4;
+  if (TI < 4) TI = 4;
+  size_t shm = (size_t)(TI + 3) * DS * 4;
 #define GC(P) hipLaunchKernelGGL((gdelta_combine_k<P>), dim3(E * H), dim3(threads), shm, st, loc, trn, ini, state, cent, H, D, TI)
   if (D <= 32) GC(32);
   else if (D <= 64) GC(64);

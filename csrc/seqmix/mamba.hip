@@ -60,7 +60,12 @@ mamba_scan_k(const float* __restrict__ conv, int C, const T* __restrict__ zx, in
   float* Sg = state + ((size_t)en.slot * H + h) * N * P;
   const bool from_state = mode == 2 || (mode == 0 && en.start > 0);
 #pragma unroll
-  for (int n = 0; n < NP; n++) S[n] = (act && n < N && from_state) ? Sg[(size_t)n * P + p] : 0.0f;
+  for (int n = 0; n < NP; n++) {
+    // loads at clamped addresses, selected afterwards: the loads stay independent of the
+    // bounds tests and go out together
+    float v = from_state ? Sg[(size_t)min(n, N - 1) * P + min(p, P - 1)] : 0.0f;
+    S[n] = (act && n < N) ? v : 0.0f;
+  }
   float A = -expf(A_log[h]), Dh = Dp[h], bias = dt_bias[h];
   float dtsum = 0.0f;
   for (int t0 = 0; t0 < en.n; t0 += CT) {
