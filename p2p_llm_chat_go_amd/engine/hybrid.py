@@ -14,6 +14,7 @@ keyed by its first page, which is unique among live sequences, and is handed bac
 """
 from __future__ import annotations
 
+import os
 import time
 
 import torch
@@ -24,11 +25,67 @@ from .engine import GenResult
 from .seq_cache import SequenceCache
 
 
+DECODE_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
+
+
+def _bucket(x: int, buckets=DECODE_BUCKETS) -> int:
+    for b in buckets:
+        if x <= b:
+            return b
+    return x
+
+
+class HybridDecodeGraph:
+    """One decode step of ``rows`` single-token entries (block tables ``maxp`` pages wide) as
+    a captured hipGraph: forward + greedy argmax.  A step loads its metadata into the batch's
+    device tensors with one copy and replays; rows beyond the live ones are padding on the
+    null page and the null state slot."""
+
+    def __init__(self, model: HybridModel, rows: int, maxp: int):
+        self.model, self.rows, self.maxp = model, rows, maxp
+        self.pad = (model.cache.null_slot, [0] * maxp, 0, [0])
+        self.batch = StepBatch([self.pad] * rows, [[0]] * rows, model.device, min_pages=maxp)
+        self.tokens = torch.zeros(rows, dtype=torch.int32, device=model.device)
+        self.logits = None
+        self.graph = None
+
+    def _body(self):
+        from .. import ops
+
+        self.logits = self.model.forward(self.batch)
+        ops.argmax(self.logits, out=self.tokens)
+
+    def capture(self, warmup: int = 2):
+        cur = torch.cuda.current_stream(self.model.device)
+        side = torch.cuda.Stream(self.model.device)
+        side.wait_stream(cur)
+        with torch.cuda.stream(side):
+            for _ in range(warmup):  # also builds everything a step creates lazily
+                self._body()
+        cur.wait_stream(side)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self._body()
+        self.graph = g
+        return self
+
+    def step(self, rows: list) -> list:
+        """rows: (slot, pages, position, token) per live sequence -> their next tokens."""
+        n = len(rows)
+        ent = [(s, list(pg) + [0] * (self.maxp - len(pg)), p, [t]) for s, pg, p, t in rows]
+        self.batch.reload(ent + [self.pad] * (self.rows - n), [[0]] * self.rows)
+        if self.batch.max_pos >= self.model.cfg.max_pos:
+            raise ValueError("position %d exceeds the model's %d positions"
+                             % (self.batch.max_pos, self.model.cfg.max_pos))
+        self.graph.replay()
+        return self.tokens[:n].cpu().tolist()
+
+
 class HybridEngine:
     def __init__(self, cfg: HybridConfig, weights: HybridWeights | None = None, device="cuda",
                  seed: int = 0, kv_pages: int | None = None, max_batch: int = 16,
                  max_prefill_tokens: int = 1024, dtype=torch.bfloat16, num_slots: int | None = None,
-                 kv_fraction: float = 0.85):
+                 kv_fraction: float = 0.85, use_graph: bool = True):
         self.cfg = cfg
         self.device = torch.device(device)
         if weights is None:
@@ -51,6 +108,11 @@ class HybridEngine:
         self.cache = self.kv = SequenceCache(specs, kv_pages, slots, self.device, self.dtype)
         self.model = HybridModel(weights, self.cache)
         self._page_slot = {}  # first page of a scheduler-owned sequence -> state slot
+        # greedy decode steps replay a captured hipGraph per (rows, table width) bucket
+        # (P2P_HYBRID_GRAPH=0: every step eager)
+        self.use_graph = (use_graph and self.device.type == "cuda"
+                          and os.environ.get("P2P_HYBRID_GRAPH", "1") != "0")
+        self._graphs = {}
 
     # ------------------------------------------------------------------ step
     def step(self, entries: list, return_layers=None):
@@ -70,6 +132,21 @@ class HybridEngine:
 
     def release(self, key):
         self.cache.close(key)
+
+    def decode_graph(self, rows: int, pages: int) -> HybridDecodeGraph:
+        key = (_bucket(rows), _bucket(pages))
+        g = self._graphs.get(key)
+        if g is None:
+            g = self._graphs[key] = HybridDecodeGraph(self.model, *key).capture()
+        return g
+
+    def _decode_rows(self, rows: list, params, pos) -> list:
+        """One token for each of rows = (slot, pages, position, token): the captured graph
+        when every row is greedy, else an eager step + the sampler."""
+        if self.use_graph and (params is None or all(p.greedy for p in params)):
+            return self.decode_graph(len(rows), max(len(r[1]) for r in rows)).step(rows)
+        b = StepBatch([(s, pg, p, [t]) for s, pg, p, t in rows], [[0]] * len(rows), self.device)
+        return self._pick(self.model.forward(b), params, pos).cpu().tolist()
 
     # ------------------------------------------------------------------ sampling
     def _pick(self, logits, params, pos):
@@ -145,9 +222,8 @@ class HybridEngine:
         ids, hist = list(last_ids), [[] for _ in last_ids]
         for j in range(k):
             rows = [(self._slot_for(block_tables[b], pos[b] + j), list(block_tables[b]), pos[b] + j,
-                     [ids[b]]) for b in range(len(ids))]
-            logits = self.model.forward(StepBatch(rows, [[0]] * len(rows), self.device))
-            ids = self._pick(logits, params, [p + j for p in pos]).cpu().tolist()
+                     ids[b]) for b in range(len(ids))]
+            ids = self._decode_rows(rows, params, [p + j for p in pos])
             for b, t in enumerate(ids):
                 hist[b].append(int(t))
         return hist
@@ -191,9 +267,14 @@ class HybridEngine:
                 if not (stop_on_eos and out[b][0] in self.cfg.eos_ids) and max_new_tokens > 1:
                     live.append(b)
             while live:
-                logits = self.step([(keys[b], [out[b][-1]], [0]) for b in live])
+                rows = []
+                for b in live:
+                    seq = self.cache.get(keys[b])
+                    self.cache.reserve(seq, seq.length + 1)
+                    rows.append((seq.slot, seq.pages, seq.length, out[b][-1]))
+                    seq.length += 1
                 prm = [sampling[b] for b in live] if sampling else None
-                toks = self._pick(logits, prm, [len(prompts[b]) + len(out[b]) - 1 for b in live]).cpu().tolist()
+                toks = self._decode_rows(rows, prm, [len(prompts[b]) + len(out[b]) - 1 for b in live])
                 nxt = []
                 for b, t in zip(live, toks):
                     out[b].append(int(t))

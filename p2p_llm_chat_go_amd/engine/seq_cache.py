@@ -64,10 +64,13 @@ class SequenceCache:
                 self.paged[i] = torch.zeros(num_pages * PAGE, int(what), device=self.device,
                                             dtype=dtype)
             elif kind == "state":
-                self.state[i] = {k: torch.zeros((num_slots,) + tuple(s), device=self.device,
+                # one slot more than the allocator hands out: the null slot, where padding rows
+                # of a bucketed (graph-captured) step keep their state, like the null page
+                self.state[i] = {k: torch.zeros((num_slots + 1,) + tuple(s), device=self.device,
                                                 dtype=torch.float32) for k, s in what.items()}
             else:
                 raise ValueError("unknown cache kind %r" % kind)
+        self.null_slot = num_slots
         self._live = {}
 
     # ------------------------------------------------------------ sequences

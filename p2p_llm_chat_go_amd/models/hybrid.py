@@ -112,9 +112,15 @@ class StepBatch:
     the position of its first token in this step and the tokens.  want: per entry the
     indices (within its tokens) whose logits are needed."""
 
-    def __init__(self, entries: list, want: list, device):
+    def __init__(self, entries: list, want: list, device, min_pages: int = 1):
+        host, meta = self.build_host(entries, want, min_pages)
+        self._adopt(host.to(device), meta)
+
+    @staticmethod
+    def build_host(entries: list, want: list, min_pages: int = 1):
+        """All of the step's metadata as one int32 host tensor + how to cut it."""
         ids, pos, row_ent, rows, ent, outs = [], [], [], [], [], []
-        maxp = max([1] + [len(e[1]) for e in entries])
+        maxp = max([min_pages] + [len(e[1]) for e in entries])
         bt = torch.zeros(len(entries), maxp, dtype=torch.int32)
         r0 = 0
         for i, (slot, pages, start, toks) in enumerate(entries):
@@ -131,24 +137,36 @@ class StepBatch:
             ent.append((r0, n, start, slot))
             outs += [r0 + w for w in want[i]]
             r0 += n
-        self.R, self.E = r0, len(entries)
-        self.ent_host = ent
-        self.n_out = len(outs)
-        self.max_pos = max(pos)
-        # one host -> device copy for all of the step's metadata
         parts = [torch.tensor(x, dtype=torch.int32).reshape(-1)
                  for x in (ids, pos, row_ent, rows, ent, outs or [0])] + [bt.reshape(-1)]
-        flat = torch.cat(parts).to(device)
-        o = 0
-        cut = []
-        for p in parts:
-            cut.append(flat[o:o + p.numel()])
-            o += p.numel()
+        meta = {"R": r0, "E": len(entries), "ent_host": ent, "n_out": len(outs),
+                "max_pos": max(pos), "maxp": maxp, "sizes": [p.numel() for p in parts]}
+        return torch.cat(parts), meta
+
+    def _adopt(self, flat, meta):
+        """flat: the device copy of ``build_host``'s tensor (one host -> device copy)."""
+        self.flat, self.meta = flat, meta
+        self.R, self.E = meta["R"], meta["E"]
+        self.ent_host, self.n_out, self.max_pos = meta["ent_host"], meta["n_out"], meta["max_pos"]
+        cut, o = [], 0
+        for n in meta["sizes"]:
+            cut.append(flat[o:o + n])
+            o += n
         self.ids, self.pos, self.row_ent, self.cache_rows = cut[0], cut[1], cut[2], cut[3]
         self.ent = cut[4].view(-1, 4)
         self.out_rows = cut[5][:self.n_out]
-        self.block_tables = cut[6].view(len(entries), maxp)
+        self.block_tables = cut[6].view(meta["E"], meta["maxp"])
         self._units = {}
+
+    def reload(self, entries: list, want: list):
+        """Same shape of step (rows, entries, wanted rows, table width), new contents, written
+        into the device tensors this batch already has (a captured graph reads them)."""
+        host, meta = self.build_host(entries, want, self.meta["maxp"])
+        if meta["sizes"] != self.meta["sizes"] or meta["maxp"] != self.meta["maxp"]:
+            raise ValueError("a reloaded step must have the shape of the captured one")
+        self.flat.copy_(host, non_blocking=True)
+        self.ent_host, self.max_pos = meta["ent_host"], meta["max_pos"]
+        self.meta = meta
 
     def units(self, rows_per_wave: int):
         """Row groups for the matrix-core attention kernel (``ops.seqmix.make_units``)."""

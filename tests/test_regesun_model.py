@@ -376,6 +376,25 @@ def test_server_scheduler_greedy(dev):
         srv.close()
 
 
+@pytest.mark.gpu
+def test_decode_graph_matches_eager():
+    """Greedy decoding through the captured step graph, replayed many times with eager steps
+    of other requests in between, gives the tokens of the eager engine."""
+    c, cfg, sd = make([GD, MB, LA, MB], seed=16)
+    prompts = [toks(n, cfg.vocab, 90 + n) for n in (70, 5, 33)]
+    w = Hy.HybridWeights(cfg, sd, "cuda:0", torch.bfloat16)
+    outs = []
+    for graph in (True, False):
+        eng = HybridEngine(cfg, w, "cuda:0", kv_pages=24, num_slots=4, max_batch=4, use_graph=graph)
+        res = eng.generate(prompts, max_new_tokens=40, stop_on_eos=False)
+        res2 = eng.generate(prompts[:2], max_new_tokens=70, stop_on_eos=False)
+        outs.append([r.tokens for r in res + res2])
+        assert bool(eng._graphs) == graph
+    assert outs[0] == outs[1]
+    for p, t in zip(prompts, outs[0]):
+        assert len(t) == 40
+
+
 def test_config_roundtrip_and_errors():
     c, cfg, sd = make([GD, MB, LA])
     assert Hy.HybridConfig.from_dict(cfg.to_dict()).layers == cfg.layers
