@@ -27,7 +27,8 @@ latent_attn_mfma_k(const bf16* __restrict__ qa, long sqh, long sqr, const bf16* 
                    const int* __restrict__ bt, int max_pages, const int* __restrict__ row_ent,
                    const int* __restrict__ pos, const int* __restrict__ units,
                    const float* __restrict__ sink, float scale, int win, bf16* __restrict__ out,
-                   long soh, long sor, int H, int rank, int page, int HS) {
+                   long soh, long sor, int H, int rank, int page, int HS, int splits,
+                   float* __restrict__ part) {
   constexpr int RP = NT2 * 32;       // padded rank
   constexpr int NT = NT2 * 2;        // 16-wide output column tiles
   constexpr int LDQ = RP + 8;
@@ -42,7 +43,16 @@ latent_attn_mfma_k(const bf16* __restrict__ qa, long sqh, long sqr, const bf16* 
   const bool pvalid = prow < nr && ph < H;
   const int ppos = pvalid ? pos[r0 + prow] : -1;
   const int* pages = bt + (size_t)row_ent[r0] * max_pages;
-  const int j_lo = max(0, pos[r0] - win + 1), j_hi = pos[r0 + nr - 1];
+  int j_lo = max(0, pos[r0] - win + 1), j_hi = pos[r0 + nr - 1];
+  if (splits > 1) {
+    // this block takes one run of 32-key tiles of the window; partial results go to `part`
+    int tiles = (j_hi - j_lo) / 32 + 1;
+    int per = (tiles + splits - 1) / splits;
+    int lo = j_lo + blockIdx.z * per * 32;
+    j_hi = min(j_hi, lo + per * 32 - 1);
+    j_lo = lo;
+  }
+  const bool first = blockIdx.z == 0;   // the sink is counted by the first run only
 
   // queries -> LDS (zero rows for unused pairs, zero columns beyond the rank)
   for (int idx = lane; idx < 16 * (RP / 8); idx += 64) {
@@ -55,8 +65,8 @@ latent_attn_mfma_k(const bf16* __restrict__ qa, long sqh, long sqr, const bf16* 
   }
   __syncthreads();
 
-  float m_run = pvalid ? sink[ph] : 0.0f;
-  float l_part = (pvalid && quad == 0) ? 1.0f : 0.0f;
+  float m_run = pvalid ? (first ? sink[ph] : -1e30f) : 0.0f;
+  float l_part = (pvalid && quad == 0 && first) ? 1.0f : 0.0f;
   f32x4 acc[NT];
 #pragma unroll
   for (int t = 0; t < NT; t++) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -144,6 +154,20 @@ latent_attn_mfma_k(const bf16* __restrict__ qa, long sqh, long sqr, const bf16* 
   }
   float l = l_part + __shfl_xor(l_part, 16, 64);
   l += __shfl_xor(l, 32, 64);
+  if (splits > 1) {
+    // partial record of this run: [pair][RP + 2] = unnormalised sums, running max, running sum
+    float* rec = part + (((size_t)blockIdx.x * gridDim.y + blockIdx.y) * splits + blockIdx.z) *
+                            16 * (RP + 2);
+    if (quad == 0) {
+      rec[n16 * (RP + 2) + RP] = m_run;
+      rec[n16 * (RP + 2) + RP + 1] = l;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+      for (int t = 0; t < NT; t++) rec[(quad * 4 + i) * (RP + 2) + t * 16 + n16] = acc[t][i];
+    return;
+  }
   float inv[4];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
@@ -165,6 +189,41 @@ latent_attn_mfma_k(const bf16* __restrict__ qa, long sqh, long sqr, const bf16* 
   }
 }
 
+// Merges the runs of a split window: out = sum_z e^(m_z - M) acc_z / sum_z e^(m_z - M) l_z.
+// One block per (unit, head group, pair); the weights of the runs are formed once in LDS.
+__global__ void latent_attn_merge_k(const float* __restrict__ part, const int* __restrict__ units,
+                                    bf16* __restrict__ out, long soh, long sor, int H, int rank,
+                                    int HS, int splits, int RP) {
+  __shared__ float sw[65];
+  const int r0 = units[2 * blockIdx.x], nr = units[2 * blockIdx.x + 1];
+  const int m = blockIdx.z;
+  const int mr = m / HS, mh = blockIdx.y * HS + m % HS;
+  if (mr >= nr || mh >= H) return;
+  const float* rec = part + ((size_t)blockIdx.x * gridDim.y + blockIdx.y) * splits * 16 * (RP + 2) +
+                     (size_t)m * (RP + 2);
+  const size_t zs = (size_t)16 * (RP + 2);   // stride between runs
+  if (threadIdx.x < 64) {
+    int z = threadIdx.x;
+    float mz = z < splits ? rec[z * zs + RP] : -INFINITY;
+    float M = mz;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
+    float w = z < splits ? expf(mz - M) : 0.0f;
+    float d = z < splits ? w * rec[z * zs + RP + 1] : 0.0f;
+    d = wave_sum(d);
+    sw[z] = w;
+    if (z == 0) sw[64] = d > 0.0f ? 1.0f / d : 0.0f;
+  }
+  __syncthreads();
+  float inv = sw[64];
+  bf16* o = out + (size_t)mh * soh + (size_t)(r0 + mr) * sor;
+  for (int c = threadIdx.x; c < rank; c += blockDim.x) {
+    float num = 0.0f;
+    for (int z = 0; z < splits; z++) num += sw[z] * rec[z * zs + c];
+    o[c] = __float2bfloat16(num * inv);
+  }
+}
+
 // the P operand's key order: slot quad*8 + i holds key quad*4 + i (i < 4) or 16 + quad*4 + i - 4;
 // the B operand above reads sC with the same order (src and src + 16).
 
@@ -180,20 +239,36 @@ int p2p_sm_latent_attn_mfma_rows(int H) {
   return 16 / hs;
 }
 
+// floats of workspace for `splits` runs per window (0 when splits <= 1)
+long p2p_sm_latent_attn_mfma_ws(int U, int H, int rank, int splits) {
+  if (splits <= 1) return 0;
+  int HS = 16 / p2p_sm_latent_attn_mfma_rows(H);
+  int n = (rank + 31) / 32;
+  int N = n <= 1 ? 1 : n <= 2 ? 2 : n <= 4 ? 4 : n <= 8 ? 8 : 16;
+  return (long)U * ((H + HS - 1) / HS) * splits * 16 * (N * 32 + 2);
+}
+
+// splits > 1: each window is cut into that many runs of key tiles (decode steps: few rows,
+// long windows), partial results in `part` (p2p_sm_latent_attn_mfma_ws floats), then merged
 int p2p_sm_latent_attn_mfma(const void* qa, long sqh, long sqr, const void* cache, const int* bt,
                             int max_pages, const int* row_ent, const int* pos, const int* units,
                             int U, const float* sink, float scale, int win, void* out, long soh,
-                            long sor, int H, int rank, int page, hipStream_t st) {
+                            long sor, int H, int rank, int page, int splits, float* part,
+                            hipStream_t st) {
   if (U <= 0) return 0;
   if (!p2p_sm_latent_attn_mfma_ok(H, rank) || win < 1) return (int)hipErrorInvalidValue;
+  if (splits < 1 || splits > 64 || (splits > 1 && !part)) return (int)hipErrorInvalidValue;
   int HS = 16 / p2p_sm_latent_attn_mfma_rows(H);
-  dim3 grid(U, (H + HS - 1) / HS), block(64);
+  dim3 grid(U, (H + HS - 1) / HS, splits), block(64);
 #define LM(N)                                                                                  \
   do {                                                                                         \
     size_t shm = (size_t)(16 * (N * 32 + 8) + N * 32 * LM_LDK) * 2;                            \
     hipLaunchKernelGGL((latent_attn_mfma_k<N>), grid, block, shm, st, (const bf16*)qa, sqh,    \
                        sqr, (const bf16*)cache, bt, max_pages, row_ent, pos, units, sink,      \
-                       scale, win, (bf16*)out, soh, sor, H, rank, page, HS);                   \
+                       scale, win, (bf16*)out, soh, sor, H, rank, page, HS, splits, part);     \
+    if (splits > 1)                                                                            \
+      hipLaunchKernelGGL(latent_attn_merge_k, dim3(grid.x, grid.y, 16), dim3(128), 0, st, part, \
+                         units, (bf16*)out, soh, sor, H, rank, HS, splits, N * 32);            \
   } while (0)
   int n = (rank + 31) / 32;
   if (n <= 1) LM(1);

@@ -45,6 +45,7 @@ class HybridDecodeGraph:
         self.model, self.rows, self.maxp = model, rows, maxp
         self.pad = (model.cache.null_slot, [0] * maxp, 0, [0])
         self.batch = StepBatch([self.pad] * rows, [[0]] * rows, model.device, min_pages=maxp)
+        self.batch.max_keys = maxp * PAGE   # a captured step must not depend on the positions
         self.tokens = torch.zeros(rows, dtype=torch.int32, device=model.device)
         self.logits = None
         self.graph = None

@@ -148,6 +148,9 @@ class StepBatch:
         self.flat, self.meta = flat, meta
         self.R, self.E = meta["R"], meta["E"]
         self.ent_host, self.n_out, self.max_pos = meta["ent_host"], meta["n_out"], meta["max_pos"]
+        # most keys any row of this step can see; a batch that is reloaded for a captured
+        # graph reports the whole width of its block tables instead
+        self.max_keys = meta["max_pos"] + 1
         cut, o = [], 0
         for n in meta["sizes"]:
             cut.append(flat[o:o + n])
@@ -318,7 +321,7 @@ class LatentAttention(Mixer):
         ol = torch.empty_like(qa)
         units = b.units(sm.latent_rows_per_wave(H)) if sm.latent_mfma_ok(qa, pool) else None
         sm.latent_attn(qa, pool, b.block_tables, b.row_ent, b.pos, self.sink, self.scale, self.win,
-                       ol, PAGE, units=units)
+                       ol, PAGE, units=units, max_keys=b.max_keys)
         o = torch.bmm(ol, self.uvt)                                                # [H, R, V]
         gated = torch.empty(b.R, H * V, device=h.device, dtype=h.dtype)
         sm.sigmoid_gate(o, proj[:, H * D + r:], gated, H, V)

@@ -57,7 +57,7 @@ _SIGS = {
                            c_int, c_int, c_int, c_int, c_void_p],
     "p2p_sm_latent_attn_mfma": [c_void_p, c_long, c_long, c_void_p, c_void_p, c_int, c_void_p,
                                 c_void_p, c_void_p, c_int, c_void_p, c_float, c_int, c_void_p,
-                                c_long, c_long, c_int, c_int, c_int, c_void_p],
+                                c_long, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
     "p2p_sm_tanh": [c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "p2p_sm_sigmoid_gate": [c_void_p, c_long, c_long, c_void_p, c_int, c_void_p, c_int, c_int,
                             c_int, c_int, c_int, c_void_p],
@@ -460,8 +460,11 @@ def latent_mfma_ok(qa, cache) -> bool:
             and cache.data_ptr() % 16 == 0 and os.environ.get("P2P_LATENT_MFMA", "1") != "0")
 
 
+LATENT_SPLIT_BLOCKS = 512   # split windows while a step has fewer blocks than this
+
+
 def latent_attn(qa, cache, block_tables, row_ent, pos, sink, scale: float, win: int, out,
-                page: int, units=None):
+                page: int, units=None, max_keys=None):
     """Windowed attention over cached latents with a softmax sink.
 
     qa [H, R, rank] (any strides, last = 1): the queries already carried into latent space
@@ -469,7 +472,8 @@ def latent_attn(qa, cache, block_tables, row_ent, pos, sink, scale: float, win: 
     at block_tables[e, t // page] * page + t % page.  out [H, R, rank] = sum_j p_j c_j with
     p = softmax over {sink_h} U {scale * qa . c_j : 0 <= pos - j < win}, the sink term having
     no value.  units: ``make_units(entries, latent_rows_per_wave(H))`` on the device; with
-    it, bf16 inputs run on the matrix cores (``latent_mfma_ok``)."""
+    it, bf16 inputs run on the matrix cores (``latent_mfma_ok``).  max_keys: an upper bound of
+    the keys any row sees (host side; lets a step of few rows split its windows)."""
     H, R, rank = qa.shape
     if not qa.is_cuda:
         bt = block_tables.long()
@@ -493,12 +497,26 @@ def latent_attn(qa, cache, block_tables, row_ent, pos, sink, scale: float, win: 
     _vec(sink, H, "sink")
     if units is not None and latent_mfma_ok(qa, cache):
         assert units.dtype == torch.int32 and units.is_contiguous() and units.shape[1] == 2
+        # few row groups with long windows (decode): cut every window into runs of key tiles
+        # so that the step fills the chip; the runs are merged by a second small kernel
+        U = units.shape[0]
+        hg = -(-H // (16 // latent_rows_per_wave(H)))
+        splits = 1
+        if max_keys is not None and U * hg < LATENT_SPLIT_BLOCKS:
+            splits = max(1, min(-(-min(max_keys, win) // 64), LATENT_SPLIT_BLOCKS // (U * hg), 64))
+        part = None
+        if splits > 1:
+            L = lib()
+            L.p2p_sm_latent_attn_mfma_ws.restype = c_long
+            n = L.p2p_sm_latent_attn_mfma_ws(U, H, rank, splits)
+            part = torch.empty(n, device=qa.device, dtype=torch.float32)
         _chk(lib().p2p_sm_latent_attn_mfma(qa.data_ptr(), qa.stride(0), qa.stride(1),
                                            cache.data_ptr(), block_tables.data_ptr(),
                                            block_tables.shape[1], row_ent.data_ptr(),
                                            pos.data_ptr(), units.data_ptr(), units.shape[0],
                                            sink.data_ptr(), scale, win, out.data_ptr(),
-                                           out.stride(0), out.stride(1), H, rank, page, _st(qa)),
+                                           out.stride(0), out.stride(1), H, rank, page, splits,
+                                           _lib.ptr(part), _st(qa)),
              "latent_attn_mfma")
         return out
     if not latent_attn_ok(H, rank):

@@ -152,3 +152,8 @@ def test_latent_attn(dt, H, rank, win):
         c = sm.latent_attn(qc, cache.to(DEV), bt.to(DEV), row_ent.to(DEV), pos.to(DEV), sink.to(DEV), 0.2,
                            win, torch.empty(H, R, rank, dtype=dt, device=DEV), page, units=units)
         torch.testing.assert_close(c.cpu().float(), a.float(), **_tol(dt))
+        # few rows, long windows: every window cut into runs of key tiles and merged
+        d = sm.latent_attn(qc, cache.to(DEV), bt.to(DEV), row_ent.to(DEV), pos.to(DEV), sink.to(DEV), 0.2,
+                           win, torch.empty(H, R, rank, dtype=dt, device=DEV), page, units=units,
+                           max_keys=140)
+        torch.testing.assert_close(d.cpu().float(), a.float(), **_tol(dt))
