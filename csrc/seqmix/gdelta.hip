@@ -126,7 +126,10 @@ gdelta_combine_k(const float* __restrict__ local, const float* __restrict__ tran
   const int DS = (D + 3) & ~3;
   int e = blockIdx.x / H, h = blockIdx.x % H;
   int c0 = cent[4 * e], nc = cent[4 * e + 1], start = cent[4 * e + 2], slot = cent[4 * e + 3];
-  int j = threadIdx.x;
+  // the block is NW groups of TD threads: every group holds all columns (thread j of a
+  // group owns column j) and takes every NW-th set of four rows
+  const int TD = ((D + 63) / 64) * 64, NW = blockDim.x / TD;
+  int j = threadIdx.x % TD, w = threadIdx.x / TD;
   bool act = j < D;
   int jc = min(j, D - 1);
   size_t DD = (size_t)D * D;
@@ -137,9 +140,10 @@ gdelta_combine_k(const float* __restrict__ local, const float* __restrict__ tran
     float v = start > 0 ? sg[(size_t)min(k, D - 1) * D + jc] : 0.0f;
     cur[k] = (act && k < D) ? v : 0.0f;
   }
+  __syncthreads();   // every group has read the slot before a single-chunk portion rewrites it
   for (int c = c0; c < c0 + nc; c++) {
     size_t off = ((size_t)c * H + h) * DD;
-    if (act) {
+    if (act && w == 0) {
 #pragma unroll
       for (int k = 0; k < DKP; k++)
         if (k < D) init[off + (size_t)k * D + j] = cur[k];
@@ -154,7 +158,7 @@ gdelta_combine_k(const float* __restrict__ local, const float* __restrict__ tran
       }
       __syncthreads();
       if (act) {
-        for (int i = 0; i < ti; i += 4) {   // four rows at a time: independent sums
+        for (int i = 4 * w; i < ti; i += 4 * NW) {   // four rows at a time: independent sums
           float a[4];
 #pragma unroll
           for (int u = 0; u < 4; u++)
@@ -175,9 +179,10 @@ gdelta_combine_k(const float* __restrict__ local, const float* __restrict__ tran
         }
       }
     }
+    __syncthreads();   // the groups' rows of the new state are all written
 #pragma unroll
     for (int k = 0; k < DKP; k++) {
-      float v = dst[(size_t)min(k, D - 1) * D + jc];   // this thread's own column, just written
+      float v = dst[(size_t)min(k, D - 1) * D + jc];   // column j, written by this block
       cur[k] = (act && k < D) ? v : 0.0f;
     }
   }
@@ -250,7 +255,8 @@ int p2p_sm_gdelta_scan_chunked(const void* r, const void* k, const void* v, cons
   if (TI > D) TI = D;
   if (TI < 4) TI = 4;
   size_t shm = (size_t)(TI + 3) * DS * 4;
-#define GC(P) hipLaunchKernelGGL((gdelta_combine_k<P>), dim3(E * H), dim3(threads), shm, st, loc, trn, ini, state, cent, H, D, TI)
+  int nw = 256 / threads;   // groups of `threads` per block
+#define GC(P) hipLaunchKernelGGL((gdelta_combine_k<P>), dim3(E * H), dim3(threads * nw), shm, st, loc, trn, ini, state, cent, H, D, TI)
   if (D <= 32) GC(32);
   else if (D <= 64) GC(64);
   else if (D <= 128) GC(128);

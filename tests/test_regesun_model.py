@@ -395,6 +395,48 @@ def test_decode_graph_matches_eager():
         assert len(t) == 40
 
 
+def test_trace_runner_cli(tmp_path):
+    """bin/trace_run on a saved checkpoint: steps on stdin, logits files and 'done' lines out,
+    finished requests hand their pages and slot back (the pool is smaller than the sum)."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+    from safetensors.torch import save_file
+
+    c, cfg, sd = make([GD, MB, LA], seed=17)
+    model = tmp_path / "model"
+    model.mkdir()
+    (model / "config.json").write_text(json.dumps(c))
+    save_file({k: v.contiguous() for k, v in sd.items()}, str(model / "model.safetensors"))
+    a, b, d = toks(90, cfg.vocab, 1), toks(40, cfg.vocab, 2), toks(100, cfg.vocab, 3)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:50], "want": [0, 49]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[50:88], "want": []},
+                                {"id": "b", "tokens": b[:39], "want": [38]}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[39:], "want": [0]},
+                                {"id": "a", "tokens": a[88:], "want": [0, 1]}], "end": ["a", "b"]},
+        {"step": 3, "entries": [{"id": "d", "tokens": d, "want": [99]}], "end": ["d"]},
+    ]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "out"
+    r = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", str(model), "--dtype", "float32",
+                        "--out", str(out), "--max-tokens", "192", "--device", "cpu"],
+                       input="".join(json.dumps(x) + "\n" for x in steps), capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [ln for ln in r.stdout.split("\n") if ln.startswith("done")] == ["done %d" % i for i in range(4)]
+    ra, rb, rd = (O.forward(c, sd, t) for t in (a, b, d))
+    got = {i: torch.from_numpy(np.fromfile(out / ("%d.f32" % i), dtype="<f4").reshape(-1, cfg.vocab))
+           for i in (0, 1, 2, 3)}
+    close(got[0], ra[[0, 49]])
+    close(got[1], rb[[38]])
+    close(got[2], torch.stack([rb[39], ra[88], ra[89]]))
+    close(got[3], rd[[99]])
+
+
 def test_config_roundtrip_and_errors():
     c, cfg, sd = make([GD, MB, LA])
     assert Hy.HybridConfig.from_dict(cfg.to_dict()).layers == cfg.layers
