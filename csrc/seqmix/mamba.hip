@@ -31,13 +31,16 @@ __global__ void mamba_conv_k(const T* __restrict__ zx, int ldz, int xoff,
   out[(size_t)r * C + c] = acc * sigmoidf_(acc);
 }
 
-template <typename T, int NP>
-__global__ void __launch_bounds__(256)
+// One thread owns NSUB consecutive state rows of one value column: thread (p, ns) holds
+// S[ns * NSUB + q][p].  Per token it updates them and leaves its share of y = S^T C in LDS;
+// the shares are added, D x and the gate applied, once per staged chunk of tokens.
+template <typename T, int NSUB>
+__global__ void __launch_bounds__(1024)
 mamba_scan_k(const float* __restrict__ conv, int C, const T* __restrict__ zx, int ldz, int xoff,
              int dtoff, const float* __restrict__ dt_bias, const float* __restrict__ A_log,
              const float* __restrict__ Dp, float* __restrict__ state, float* __restrict__ tail,
              const int* __restrict__ ent, float* __restrict__ y, int H, int P, int N, int G,
-             int K, int CT, int mode, float* __restrict__ decay_out) {
+             int K, int CT, int mode, float* __restrict__ decay_out, int TP, int NS) {
   // mode 0: a portion from its slot's state (or zero at position 0), state written back.
   // mode 1: a chunk from a zero state: no outputs; the end state goes to `state[slot]` and
   //         the product of the chunk's decays to decay_out[entry, head].
@@ -46,32 +49,36 @@ mamba_scan_k(const float* __restrict__ conv, int C, const T* __restrict__ zx, in
   Entry en = load_entry(ent, e);
   if (en.n <= 0) return;
   extern __shared__ float smem[];
-  float* sB = smem;                // [CT][NP]
-  float* sC = sB + CT * NP;        // [CT][NP]
-  float* sx = sC + CT * NP;        // [CT][P]
-  float* sz = sx + CT * P;         // [CT][P]
-  float* sdt = sz + CT * P;        // [CT]
-  float* sdA = sdt + CT;           // [CT]
+  const int NPAD = NS * NSUB;
+  float* sB = smem;                  // [CT][NPAD]
+  float* sC = sB + CT * NPAD;        // [CT][NPAD]
+  float* sx = sC + CT * NPAD;        // [CT][P]
+  float* sz = sx + CT * P;           // [CT][P]
+  float* sy = sz + CT * P;           // [CT][NS][P] shares of y
+  float* sdt = sy + CT * NS * P;     // [CT]
+  float* sdA = sdt + CT;             // [CT]
   int inner = H * P;
   int g = h / (H / G);
-  int p = threadIdx.x;
-  bool act = p < P;
-  float S[NP];
+  const int p = threadIdx.x % TP, ns = threadIdx.x / TP;
+  const bool act = p < P;
+  const int n0 = ns * NSUB;
+  float S[NSUB];
   float* Sg = state + ((size_t)en.slot * H + h) * N * P;
   const bool from_state = mode == 2 || (mode == 0 && en.start > 0);
 #pragma unroll
-  for (int n = 0; n < NP; n++) {
+  for (int q = 0; q < NSUB; q++) {
     // loads at clamped addresses, selected afterwards: the loads stay independent of the
     // bounds tests and go out together
-    float v = from_state ? Sg[(size_t)min(n, N - 1) * P + min(p, P - 1)] : 0.0f;
-    S[n] = (act && n < N) ? v : 0.0f;
+    float v = from_state ? Sg[(size_t)min(n0 + q, N - 1) * P + min(p, P - 1)] : 0.0f;
+    S[q] = (act && n0 + q < N) ? v : 0.0f;
   }
   float A = -expf(A_log[h]), Dh = Dp[h], bias = dt_bias[h];
   float dtsum = 0.0f;
   for (int t0 = 0; t0 < en.n; t0 += CT) {
     int ct = min(CT, en.n - t0);
-    for (int idx = threadIdx.x; idx < ct * NP; idx += blockDim.x) {
-      int t = idx / NP, n = idx % NP;
+    __syncthreads();   // the previous chunk's outputs have been read
+    for (int idx = threadIdx.x; idx < ct * NPAD; idx += blockDim.x) {
+      int t = idx / NPAD, n = idx % NPAD;
       size_t row = (size_t)(en.row0 + t0 + t);
       float b = 0.f, c = 0.f;
       if (n < N) {
@@ -95,28 +102,38 @@ mamba_scan_k(const float* __restrict__ conv, int C, const T* __restrict__ zx, in
     __syncthreads();
     if (act) {
       for (int t = 0; t < ct; t++) {
-        float dA = sdA[t], xp = sx[t * P + p];
+        float dA = sdA[t];
+        float dx = sdt[t] * sx[t * P + p];
         dtsum += sdt[t];
-        float dx = sdt[t] * xp;
+        const float* bb = sB + t * NPAD + n0;
+        const float* cc = sC + t * NPAD + n0;
         float acc = 0.0f;
 #pragma unroll
-        for (int n = 0; n < NP; n++) {
-          S[n] = dA * S[n] + dx * sB[t * NP + n];
-          acc += S[n] * sC[t * NP + n];
+        for (int q = 0; q < NSUB; q++) {
+          S[q] = dA * S[q] + dx * bb[q];
+          acc += S[q] * cc[q];
         }
-        acc += Dh * xp;
-        float z = sz[t * P + p];
-        if (mode != 1) y[(size_t)(en.row0 + t0 + t) * inner + h * P + p] = acc * (z * sigmoidf_(z));
+        sy[(t * NS + ns) * P + p] = acc;
       }
     }
     __syncthreads();
+    if (mode != 1) {
+      for (int idx = threadIdx.x; idx < ct * P; idx += blockDim.x) {
+        int t = idx / P, q = idx % P;
+        float acc = 0.0f;
+        for (int k = 0; k < NS; k++) acc += sy[(t * NS + k) * P + q];
+        acc += Dh * sx[idx];
+        float z = sz[idx];
+        y[(size_t)(en.row0 + t0 + t) * inner + h * P + q] = acc * (z * sigmoidf_(z));
+      }
+    }
   }
   if (act && mode != 2) {
 #pragma unroll
-    for (int n = 0; n < NP; n++)
-      if (n < N) Sg[(size_t)n * P + p] = S[n];
+    for (int q = 0; q < NSUB; q++)
+      if (n0 + q < N) Sg[(size_t)(n0 + q) * P + p] = S[q];
   }
-  if (mode == 1 && p == 0) decay_out[(size_t)e * H + h] = expf(A * dtsum);
+  if (mode == 1 && threadIdx.x == 0) decay_out[(size_t)e * H + h] = expf(A * dtsum);
 }
 
 // Chains the chunks of each portion: chunk c starts from init_c, init_{c+1} = decay_c * init_c
@@ -160,20 +177,21 @@ __global__ void mamba_tail_k(const T* __restrict__ zx, int ldz, int xoff, float*
   }
 }
 
-template <typename T, int NP>
+template <typename T, int NSUB>
 static int launch_ms(const float* conv, int C, const void* zx, int ldz, int xoff, int dtoff,
                      const float* dt_bias, const float* A_log, const float* Dp, float* state,
                      float* tail, const int* ent, int E, float* y, int H, int P, int N, int G,
                      int K, int mode, float* decay_out, hipStream_t st) {
-  int threads = ((P + 63) / 64) * 64;
-  int per = 2 * NP + 2 * P + 2;
+  int TP = ((P + 63) / 64) * 64;
+  int NS = (N + NSUB - 1) / NSUB;
+  int per = 2 * NS * NSUB + 2 * P + NS * P + 2;
   int CT = (48 * 1024) / (per * 4);
   if (CT > 32) CT = 32;
   if (CT < 1) CT = 1;
   size_t shm = (size_t)CT * per * 4;
-  hipLaunchKernelGGL((mamba_scan_k<T, NP>), dim3(E * H), dim3(threads), shm, st, conv, C,
+  hipLaunchKernelGGL((mamba_scan_k<T, NSUB>), dim3(E * H), dim3(TP * NS), shm, st, conv, C,
                      (const T*)zx, ldz, xoff, dtoff, dt_bias, A_log, Dp, state, tail, ent, y, H,
-                     P, N, G, K, CT, mode, decay_out);
+                     P, N, G, K, CT, mode, decay_out, TP, NS);
   return (int)hipGetLastError();
 }
 
@@ -200,10 +218,11 @@ int p2p_sm_mamba_scan_mode(const float* conv, int C, const void* zx, int ldz, in
   SM_DISPATCH_T(f32, return (launch_ms<T, NPV>(conv, C, zx, ldz, xoff, dtoff, dt_bias, A_log, \
                                                Dp, state, tail, ent, E, y, H, P, N, G, K, mode, \
                                                decay_out, st)))
-  if (N <= 32) MS(32);
-  else if (N <= 64) MS(64);
-  else if (N <= 128) MS(128);
-  else MS(256);
+  // state rows per thread: 32 where the block (value columns x row slices) fits 1024 threads
+  int TPv = ((P + 63) / 64) * 64;
+  // (value and state sizes are at most 256, so 64 rows per thread always fit)
+  if (TPv * ((N + 31) / 32) <= 1024) MS(32);
+  else MS(64);
 #undef MS
   return 0;
 }

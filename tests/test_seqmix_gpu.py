@@ -102,7 +102,7 @@ def test_gdelta(dt, H, D, scan_chunk):
 
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,P,N,G,K", [(6, 40, 24, 3, 3), (4, 24, 16, 1, 4), (2, 72, 80, 2, 2)])
+@pytest.mark.parametrize("H,P,N,G,K", [(6, 40, 24, 3, 3), (4, 24, 16, 1, 4), (2, 72, 80, 2, 2), (2, 200, 256, 1, 4), (8, 64, 128, 4, 4)])
 def test_mamba(dt, H, P, N, G, K, scan_chunk):
     g = torch.Generator().manual_seed(3)
     inner, C = H * P, H * P + 2 * G * N
