@@ -10,8 +10,12 @@ using namespace sm;
 
 #define GD_DECAY_SCALE 0.6065306597126334f  // exp(-1/2)
 
-template <typename T, int DKP>
-__global__ void __launch_bounds__(256)
+// Thread layout: a wavefront covers 16 value columns x 4 slices of the key index; lane
+// (c, s) holds rows s * DQ .. s * DQ + DQ - 1 of column c.  The two sums a token needs over
+// the whole key index (|k|^2 and u^T S before the update, S^T r after it) are finished with
+// two lane shuffles, so a token costs DQ steps instead of D.
+template <typename T, int DQ>
+__global__ void __launch_bounds__(1024)
 gdelta_scan_k(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v,
               const T* __restrict__ g, const T* __restrict__ a, int ld,
               const T* __restrict__ lo, int ldlo, const float* __restrict__ w0,
@@ -23,6 +27,7 @@ gdelta_scan_k(const T* __restrict__ r, const T* __restrict__ k, const T* __restr
   //         end state in state[slot]; blockIdx.y = 1 runs only the state transition on the
   //         identity (no k v^T term) and leaves the chunk's transition matrix in state2[slot].
   // mode 2: a chunk from state[slot], outputs only.
+  constexpr int DKP = 4 * DQ;   // padded key index (zero filled in LDS)
   int e = blockIdx.x / H, h = blockIdx.x % H;
   const bool trans = mode == 1 && blockIdx.y == 1;
   Entry en = load_entry(ent, e);
@@ -34,20 +39,21 @@ gdelta_scan_k(const T* __restrict__ r, const T* __restrict__ k, const T* __restr
   float* sw = sv + CT * DKP;
   float* sa = sw + CT * DKP;
   float* so = sa + CT * DKP;
-  int j = threadIdx.x;
-  bool act = j < D;
-  float S[DKP];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const int j = wave * 16 + (lane & 15), is = lane >> 4, i0 = is * DQ;
+  const bool act = j < D;
+  const int jc = min(j, D - 1);
+  float S[DQ];
   float* Sg = (trans ? state2 : state) + ((size_t)en.slot * H + h) * D * D;
   const bool from_state = mode == 2 || (mode == 0 && en.start > 0);
 #pragma unroll
-  for (int i = 0; i < DKP; i++) {
+  for (int q = 0; q < DQ; q++) {
     // loads at clamped addresses, selected afterwards: the loads stay independent of the
     // bounds tests and go out together
-    float v0 = trans ? (i == j ? 1.0f : 0.0f) : 0.0f;
-    float v = from_state ? Sg[(size_t)min(i, D - 1) * D + min(j, D - 1)] : v0;
-    S[i] = (act && i < D) ? v : 0.0f;
+    float v0 = (trans && i0 + q == j) ? 1.0f : 0.0f;
+    float vv = from_state ? Sg[(size_t)min(i0 + q, D - 1) * D + jc] : v0;
+    S[q] = (act && i0 + q < D) ? vv : 0.0f;
   }
-  int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   for (int t0 = 0; t0 < en.n; t0 += CT) {
     int ct = min(CT, en.n - t0);
     for (int idx = threadIdx.x; idx < ct * DKP; idx += blockDim.x) {
@@ -65,29 +71,33 @@ gdelta_scan_k(const T* __restrict__ r, const T* __restrict__ k, const T* __restr
       sr[idx] = vr; sk[idx] = vk; sv[idx] = vv; sw[idx] = vw; sa[idx] = va;
     }
     __syncthreads();
-    if (act) {
-      for (int t = 0; t < ct; t++) {
-        const float* kr = sk + t * DKP;
-        float kk = 0.0f, d = 0.0f;
+    for (int t = 0; t < ct; t++) {   // every lane takes part (the shuffles need all of them)
+      const float* kr = sk + t * DKP + i0;
+      float kk = 0.0f, d = 0.0f;
 #pragma unroll
-        for (int i = 0; i < DKP; i++) {
-          float ki = kr[i];
-          kk += ki * ki;
-          d += ki * S[i];
-        }
-        float rs = 1.0f / sqrtf(kk + 1e-6f);
-        float dot = d * rs;            // u^T S (column j)
-        float vj = trans ? 0.0f : sv[t * DKP + j];
-        float o = 0.0f;
-#pragma unroll
-        for (int i = 0; i < DKP; i++) {
-          float ki = kr[i];
-          float ui = ki * rs;
-          S[i] = sw[t * DKP + i] * S[i] - (sa[t * DKP + i] * ui) * dot + ki * vj;
-          o += S[i] * sr[t * DKP + i];
-        }
-        so[t * DKP + j] = o;
+      for (int q = 0; q < DQ; q++) {
+        float ki = kr[q];
+        kk += ki * ki;
+        d += ki * S[q];
       }
+      kk += __shfl_xor(kk, 16, 64);
+      d += __shfl_xor(d, 16, 64);
+      kk += __shfl_xor(kk, 32, 64);
+      d += __shfl_xor(d, 32, 64);
+      float rs = 1.0f / sqrtf(kk + 1e-6f);
+      float dot = d * rs;            // u^T S (column j)
+      float vj = trans ? 0.0f : sv[t * DKP + jc];
+      float o = 0.0f;
+#pragma unroll
+      for (int q = 0; q < DQ; q++) {
+        float ki = kr[q];
+        float ui = ki * rs;
+        S[q] = sw[t * DKP + i0 + q] * S[q] - (sa[t * DKP + i0 + q] * ui) * dot + ki * vj;
+        o += S[q] * sr[t * DKP + i0 + q];
+      }
+      o += __shfl_xor(o, 16, 64);
+      o += __shfl_xor(o, 32, 64);
+      if (is == 0 && act) so[t * DKP + j] = o;
     }
     __syncthreads();
     if (mode != 1)
@@ -109,8 +119,8 @@ gdelta_scan_k(const T* __restrict__ r, const T* __restrict__ k, const T* __restr
   }
   if (act && mode != 2) {
 #pragma unroll
-    for (int i = 0; i < DKP; i++)
-      if (i < D) Sg[(size_t)i * D + j] = S[i];
+    for (int q = 0; q < DQ; q++)
+      if (i0 + q < D) Sg[(size_t)(i0 + q) * D + j] = S[q];
   }
 }
 
@@ -188,17 +198,18 @@ gdelta_combine_k(const float* __restrict__ local, const float* __restrict__ tran
   }
 }
 
-template <typename T, int DKP>
+template <typename T, int DQ>
 static int launch_gd(const void* r, const void* k, const void* v, const void* g, const void* a,
                      int ld, const void* lo, int ldlo, const float* w0, const float* ab,
                      const float* normw, float* state, const int* ent, int E, void* out, int ldo,
                      int H, int D, float eps, int mode, float* state2, hipStream_t st) {
-  int threads = ((D + 63) / 64) * 64;
+  constexpr int DKP = 4 * DQ;
+  int threads = ((D + 15) / 16) * 64;   // a wavefront per 16 value columns
   int CT = (48 * 1024) / (6 * DKP * 4);
   if (CT > 32) CT = 32;
   if (CT < 1) CT = 1;
   size_t shm = (size_t)6 * CT * DKP * 4;
-  hipLaunchKernelGGL((gdelta_scan_k<T, DKP>), dim3(E * H, mode == 1 ? 2 : 1), dim3(threads), shm,
+  hipLaunchKernelGGL((gdelta_scan_k<T, DQ>), dim3(E * H, mode == 1 ? 2 : 1), dim3(threads), shm,
                      st, (const T*)r, (const T*)k, (const T*)v, (const T*)g, (const T*)a, ld,
                      (const T*)lo, ldlo, w0, ab, normw, state, ent, (T*)out, ldo, H, D, eps, CT,
                      mode, state2);
@@ -217,10 +228,10 @@ int p2p_sm_gdelta_scan_mode(const void* r, const void* k, const void* v, const v
 #define GD(P)                                                                                   \
   SM_DISPATCH_T(f32, return (launch_gd<T, P>(r, k, v, g, a, ld, lo, ldlo, w0, ab, normw, state, \
                                              ent, E, out, ldo, H, D, eps, mode, state2, st)))
-  if (D <= 32) GD(32);
-  else if (D <= 64) GD(64);
-  else if (D <= 128) GD(128);
-  else GD(256);
+  if (D <= 32) GD(8);
+  else if (D <= 64) GD(16);
+  else if (D <= 128) GD(32);
+  else GD(64);
 #undef GD
   return 0;
 }

@@ -80,7 +80,7 @@ def scan_chunk(request, monkeypatch):
 
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,D", [(2, 40), (3, 20), (1, 72)])
+@pytest.mark.parametrize("H,D", [(2, 40), (3, 20), (1, 72), (2, 64), (1, 136), (2, 7)])
 def test_gdelta(dt, H, D, scan_chunk):
     g = torch.Generator().manual_seed(2)
     n = H * D
