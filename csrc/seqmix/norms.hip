@@ -17,6 +17,8 @@ __global__ void embed_pos_k(const T* __restrict__ embed, const T* __restrict__ p
   }
 }
 
+#define NV 16   // values a thread keeps in registers: rows of up to 256 * NV numbers are read once
+
 // one block per (row, part): out = x / sqrt(mean(x^2) + eps) * w
 template <typename TI, typename TO>
 __global__ void rmsnorm_k(const TI* __restrict__ x, int ldx, const float* __restrict__ w,
@@ -26,20 +28,43 @@ __global__ void rmsnorm_k(const TI* __restrict__ x, int ldx, const float* __rest
   int r = blockIdx.x / parts, g = blockIdx.x % parts;
   int np = n / parts;
   int ri = in_rows ? in_rows[r] : r;
+  int ro = out_rows ? out_rows[r] : r;
   const TI* xr = x + (size_t)ri * ldx + (size_t)g * np;
+  const float* wp = w ? w + g * np : nullptr;
+  if (np <= NV * (int)blockDim.x) {
+    // the row and its weights are loaded once, before the reduction
+    float v[NV], wv[NV];
+    float ss = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+      int i = threadIdx.x + k * blockDim.x;
+      v[k] = i < np ? ldf(xr, i) : 0.0f;
+      wv[k] = (wp && i < np) ? wp[i] : 1.0f;
+      ss += v[k] * v[k];
+    }
+    ss = block_sum(ss, red);
+    if (ro < 0) return;
+    float rs = 1.0f / sqrtf(ss / (float)np + eps);
+    TO* o = out + (size_t)ro * ldo + (size_t)g * np;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+      int i = threadIdx.x + k * blockDim.x;
+      if (i < np) stf(o, i, v[k] * rs * wv[k]);
+    }
+    return;
+  }
   float ss = 0.0f;
   for (int i = threadIdx.x; i < np; i += blockDim.x) {
     float v = ldf(xr, i);
     ss += v * v;
   }
   ss = block_sum(ss, red);
-  int ro = out_rows ? out_rows[r] : r;
   if (ro < 0) return;
   float rs = 1.0f / sqrtf(ss / (float)np + eps);
   TO* o = out + (size_t)ro * ldo + (size_t)g * np;
   for (int i = threadIdx.x; i < np; i += blockDim.x) {
     float v = ldf(xr, i) * rs;
-    if (w) v *= w[g * np + i];
+    if (wp) v *= wp[i];
     stf(o, i, v);
   }
 }
@@ -52,6 +77,29 @@ __global__ void norm_scale_add_k(float* __restrict__ x, const T* __restrict__ y,
   __shared__ float red[16];
   int r = blockIdx.x;
   const T* yr = y + (size_t)r * ldy;
+  float* xr = x + (size_t)r * n;
+  if (n <= NV * (int)blockDim.x) {
+    // y, the weights and the residual are loaded once, before the reduction
+    float v[NV], wv[NV], xv[NV];
+    float ss = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+      int i = threadIdx.x + k * blockDim.x;
+      bool ok = i < n;
+      v[k] = ok ? ldf(yr, i) : 0.0f;
+      wv[k] = ok ? (ls ? w[i] * ls[i] : w[i]) : 0.0f;
+      xv[k] = ok ? xr[i] : 0.0f;
+      ss += v[k] * v[k];
+    }
+    ss = block_sum(ss, red);
+    float rs = 1.0f / sqrtf(ss / (float)n + eps);
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+      int i = threadIdx.x + k * blockDim.x;
+      if (i < n) xr[i] = xv[k] + v[k] * rs * wv[k];
+    }
+    return;
+  }
   float ss = 0.0f;
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
     float v = ldf(yr, i);
@@ -60,9 +108,8 @@ __global__ void norm_scale_add_k(float* __restrict__ x, const T* __restrict__ y,
   ss = block_sum(ss, red);
   float rs = 1.0f / sqrtf(ss / (float)n + eps);
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
-    float v = ldf(yr, i) * rs * w[i];
-    if (ls) v *= ls[i];
-    x[(size_t)r * n + i] += v;
+    float v = ldf(yr, i) * rs * (ls ? w[i] * ls[i] : w[i]);
+    xr[i] += v;
   }
 }
 
