@@ -69,11 +69,13 @@ __global__ void rmsnorm_k(const TI* __restrict__ x, int ldx, const float* __rest
   }
 }
 
-// x += y / sqrt(mean(y^2) + eps) * w * ls   (x fp32 residual)
+// x += y / sqrt(mean(y^2) + eps) * w * ls   (x fp32 residual); with w2 also the next
+// sublayer's input h = x / sqrt(mean(x^2) + eps) * w2 from the updated row
 template <typename T>
 __global__ void norm_scale_add_k(float* __restrict__ x, const T* __restrict__ y, int ldy,
                                  const float* __restrict__ w, const float* __restrict__ ls,
-                                 int n, float eps) {
+                                 int n, float eps, const float* __restrict__ w2,
+                                 T* __restrict__ h, int ldh) {
   __shared__ float red[16];
   int r = blockIdx.x;
   const T* yr = y + (size_t)r * ldy;
@@ -93,10 +95,21 @@ __global__ void norm_scale_add_k(float* __restrict__ x, const T* __restrict__ y,
     }
     ss = block_sum(ss, red);
     float rs = 1.0f / sqrtf(ss / (float)n + eps);
+    float s2 = 0.0f;
 #pragma unroll
     for (int k = 0; k < NV; k++) {
       int i = threadIdx.x + k * blockDim.x;
-      if (i < n) xr[i] = xv[k] + v[k] * rs * wv[k];
+      xv[k] = xv[k] + v[k] * rs * wv[k];
+      if (i < n) xr[i] = xv[k];
+      s2 += xv[k] * xv[k];
+    }
+    if (!w2) return;
+    s2 = block_sum(s2, red);
+    float r2 = 1.0f / sqrtf(s2 / (float)n + eps);
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+      int i = threadIdx.x + k * blockDim.x;
+      if (i < n) stf(h, (size_t)r * ldh + i, xv[k] * r2 * w2[i]);
     }
     return;
   }
@@ -107,10 +120,17 @@ __global__ void norm_scale_add_k(float* __restrict__ x, const T* __restrict__ y,
   }
   ss = block_sum(ss, red);
   float rs = 1.0f / sqrtf(ss / (float)n + eps);
+  float s2 = 0.0f;
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
-    float v = ldf(yr, i) * rs * (ls ? w[i] * ls[i] : w[i]);
-    xr[i] += v;
+    float v = xr[i] + ldf(yr, i) * rs * (ls ? w[i] * ls[i] : w[i]);
+    xr[i] = v;
+    s2 += v * v;
   }
+  if (!w2) return;
+  s2 = block_sum(s2, red);
+  float r2 = 1.0f / sqrtf(s2 / (float)n + eps);
+  for (int i = threadIdx.x; i < n; i += blockDim.x)   // each thread re-reads its own writes
+    stf(h, (size_t)r * ldh + i, xr[i] * r2 * w2[i]);
 }
 
 extern "C" {
@@ -142,10 +162,11 @@ int p2p_sm_rmsnorm(const void* x, int ldx, int in_f32, const float* w, void* out
 }
 
 int p2p_sm_norm_scale_add(float* x, const void* y, int ldy, const float* w, const float* ls,
-                          int R, int n, float eps, int f32, hipStream_t st) {
+                          int R, int n, float eps, const float* w2, void* h, int ldh, int f32,
+                          hipStream_t st) {
   if (R <= 0) return 0;
   SM_DISPATCH_T(f32, hipLaunchKernelGGL(norm_scale_add_k<T>, dim3(R), dim3(256), 0, st, x,
-                                         (const T*)y, ldy, w, ls, n, eps));
+                                         (const T*)y, ldy, w, ls, n, eps, w2, (T*)h, ldh));
   return (int)hipGetLastError();
 }
 

@@ -467,13 +467,17 @@ class HybridModel:
         x = torch.empty(b.R, cfg.width, device=self.device, dtype=torch.float32)
         sm.embed_pos(w.embed, w.pos, b.ids, b.pos, x)
         h = torch.empty(b.R, cfg.width, device=self.device, dtype=self.dtype)
+        # every post-sublayer pass (norm, layer scale, residual add) also forms the next
+        # sublayer's normed input from the updated rows
+        sm.rmsnorm(x, w.layers[0].norm1, cfg.eps, h)
         for i, L in enumerate(w.layers):
-            sm.rmsnorm(x, L.norm1, cfg.eps, h)
+            after = w.layers[i + 1].norm1 if i + 1 < len(w.layers) else None
             m = L.mixer.forward(h, b, self.cache, i)
-            sm.norm_scale_add(x, m, L.norm1b, L.ls1, cfg.eps)
+            sm.norm_scale_add(x, m, L.norm1b, L.ls1, cfg.eps,
+                              next_w=L.norm2 if L.ff is not None else after, next_out=h)
             if L.ff is not None:
-                sm.rmsnorm(x, L.norm2, cfg.eps, h)
-                sm.norm_scale_add(x, L.ff.forward(h), L.norm2b, L.ls2, cfg.eps)
+                sm.norm_scale_add(x, L.ff.forward(h), L.norm2b, L.ls2, cfg.eps, next_w=after,
+                                  next_out=h)
             if layer_out is not None:
                 layer_out.append(x.clone())
         if b.n_out == 0:

@@ -33,7 +33,7 @@ _SIGS = {
     "p2p_sm_rmsnorm": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                        c_void_p, c_int, c_int, c_int, c_float, c_void_p],
     "p2p_sm_norm_scale_add": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int,
-                              c_float, c_int, c_void_p],
+                              c_float, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "p2p_sm_gdelta_scan": [c_void_p] * 5 + [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                                             c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
                                             c_int, c_float, c_int, c_void_p],
@@ -193,22 +193,34 @@ def rmsnorm(x, w, eps, out, parts: int = 1, in_rows=None, out_rows=None):
     return out
 
 
-def norm_scale_add(x, y, w, ls, eps):
-    """x += y / sqrt(mean(y^2) + eps) * w * ls on the fp32 residual x (ls may be None)."""
+def norm_scale_add(x, y, w, ls, eps, next_w=None, next_out=None):
+    """x += y / sqrt(mean(y^2) + eps) * w * ls on the fp32 residual x (ls may be None).
+    With next_w / next_out also the next sublayer's input in the same pass:
+    next_out = x / sqrt(mean(x^2) + eps) * next_w from the updated rows."""
     R, n = x.shape
     if not x.is_cuda:
         v = _rms(y.float(), eps) * w
         if ls is not None:
             v = v * ls
         x += v
+        if next_w is not None:
+            next_out[:R] = (_rms(x, eps) * next_w).to(next_out.dtype)
         return x
     _rows2d(y, "y")
     assert x.dtype == torch.float32 and x.is_contiguous() and y.shape == x.shape
     _vec(w, n, "w")
     if ls is not None:
         _vec(ls, n, "ls")
+    ldh = 0
+    if next_w is not None:
+        _vec(next_w, n, "next_w")
+        _rows2d(next_out, "next_out")
+        assert next_out.dtype == y.dtype and next_out.shape[1] == n and next_out.shape[0] >= R
+        ldh = next_out.stride(0)
     _chk(lib().p2p_sm_norm_scale_add(x.data_ptr(), y.data_ptr(), y.stride(0), w.data_ptr(),
-                                     _lib.ptr(ls), R, n, eps, _f32(y), _st(x)), "norm_scale_add")
+                                     _lib.ptr(ls), R, n, eps, _lib.ptr(next_w),
+                                     _lib.ptr(next_out if next_w is not None else None), ldh,
+                                     _f32(y), _st(x)), "norm_scale_add")
     return x
 
 

@@ -24,9 +24,10 @@ def _tol(dt):
 
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
-def test_embed_norms(dt):
+@pytest.mark.parametrize("wide", [200, 4100])   # rows kept in registers / rows read twice
+def test_embed_norms(dt, wide):
     g = torch.Generator().manual_seed(0)
-    V, W, R = 50, 200, 37
+    V, W, R = 50, wide, 37
     emb, ptab = torch.randn(V, W, generator=g).to(dt), torch.randn(64, W, generator=g).to(dt)
     ids = torch.randint(0, V, (R,), generator=g, dtype=torch.int32)
     pos = torch.randint(0, 64, (R,), generator=g, dtype=torch.int32)
@@ -34,7 +35,7 @@ def test_embed_norms(dt):
     b = sm.embed_pos(emb.to(DEV), ptab.to(DEV), ids.to(DEV), pos.to(DEV), torch.empty(R, W, device=DEV))
     torch.testing.assert_close(b.cpu(), a, rtol=0, atol=0)
     w = torch.randn(W, generator=g)
-    for parts in (1, 4):
+    for parts in (1, 4) if wide % 4 == 0 else (1,):
         o1 = sm.rmsnorm(a, w, 1e-5, torch.empty(R, W, dtype=dt), parts=parts)
         o2 = sm.rmsnorm(b, w.to(DEV), 1e-5, torch.empty(R, W, dtype=dt, device=DEV), parts=parts)
         torch.testing.assert_close(o2.cpu().float(), o1.float(), **_tol(dt))
@@ -50,6 +51,13 @@ def test_embed_norms(dt):
     x1 = sm.norm_scale_add(a.clone(), y, w, ls, 1e-5)
     x2 = sm.norm_scale_add(b.clone(), y.to(DEV), w.to(DEV), ls.to(DEV), 1e-5)
     torch.testing.assert_close(x2.cpu(), x1, rtol=1e-5, atol=1e-5)
+    # ... and the next sublayer's normed input in the same pass
+    w2 = torch.randn(W, generator=g)
+    h1, h2 = torch.empty(R, W, dtype=dt), torch.empty(R, W, dtype=dt, device=DEV)
+    x1 = sm.norm_scale_add(a.clone(), y, w, ls, 1e-5, next_w=w2, next_out=h1)
+    x2 = sm.norm_scale_add(b.clone(), y.to(DEV), w.to(DEV), ls.to(DEV), 1e-5, next_w=w2.to(DEV), next_out=h2)
+    torch.testing.assert_close(x2.cpu(), x1, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(h2.cpu().float(), h1.float(), **_tol(dt))
 
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
