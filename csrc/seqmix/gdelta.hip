@@ -1,10 +1,11 @@
 // Generalized delta rule: per head a D x D fp32 state S (key index i, value index j),
 //   S <- diag(w) S - (a * u)(u^T S) + k v^T,   o = S^T r,   u = k / sqrt(|k|^2 + 1e-6),
-// decay and removal both applied to the state as it was before the token.  Value columns are independent, so one thread
-// owns column j of S in registers and walks the tokens of its sequence portion in order;
-// the per-token vectors (r, k, v, decay w, removal rate a) are staged through LDS a chunk
-// of tokens at a time, with the decay and the rate evaluated while staging.  The head's
-// outputs are RMS-normalised, weighted and gated as each chunk finishes.
+// decay and removal both applied to the state as it was before the token.  The value columns
+// of S are independent; the state sits in registers and the tokens of a sequence portion are
+// walked in order.  The per-token vectors (r, k, v, decay w, removal rate a) are staged
+// through LDS a chunk of tokens at a time, with the decay and the rate evaluated while
+// staging.  The head's outputs are RMS-normalised, weighted and gated as each chunk
+// finishes.  Long portions run as chunks side by side (modes 1 and 2 + gdelta_combine_k).
 #include "common.h"
 using namespace sm;
 

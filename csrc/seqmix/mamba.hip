@@ -3,8 +3,10 @@
 //          before a portion's first token come from the sequence's saved tail (the last
 //          taps-1 raw inputs), or are zero at the start of a sequence.
 //   scan : per head an N x P fp32 state, S <- exp(-exp(A_log) dt) S + dt B x^T,
-//          y = S^T C + D x, y *= silu(z); dt = softplus(raw + bias).  One thread owns value
-//          column p of S in registers; B, C, x, z, dt of a chunk of tokens go through LDS.
+//          y = S^T C + D x, y *= silu(z); dt = softplus(raw + bias).  The state sits in
+//          registers (a thread holds a run of state rows of one value column); B, C, x, z,
+//          dt of a chunk of tokens go through LDS.  Long portions run as chunks side by
+//          side (modes 1 and 2 + mamba_combine_k).
 //   tail : rolls the convolution tail forward after the scan.
 #include "common.h"
 using namespace sm;
