@@ -1,3 +1,4 @@
 from .engine import Engine, GenResult
+from .hybrid import HybridEngine
 
-__all__ = ["Engine", "GenResult"]
+__all__ = ["Engine", "GenResult", "HybridEngine"]
