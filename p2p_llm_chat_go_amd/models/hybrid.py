@@ -288,7 +288,7 @@ class LatentAttention(Mixer):
         s = self.spec
         self.H, self.D, self.V, self.rank = int(s["heads"]), int(s["dim"]), int(s["vdim"]), int(s["kv_rank"])
         self.win = int(s["mask"]["size"]) if s.get("mask") else 1 << 30
-        self.scale = float(s["scale"])
+        self.scale = float(s["scale"]) if "scale" in s else self.D ** -0.5
 
     def tensor_shapes(self):
         self._dims()

@@ -6,8 +6,6 @@ in float32 (and bfloat16 with a loose bound).  The CPU variants exercise the mod
 batching and scheduling code with the ops' PyTorch rendering; the ``gpu`` variants run the
 same cases on the HIP kernels.
 """
-import math
-
 import pytest
 import torch
 
