@@ -19,7 +19,8 @@ using namespace sm;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-#define LM_LDK 40   // keys per transposed row in LDS (32 + padding), in bf16
+#define LM_LDK 36   // keys per transposed row in LDS (32 + padding), in bf16: rows 72 bytes apart
+                    // spread the four key-index slices over different banks
 
 template <int NT2>  // rank padded to NT2 * 32
 __global__ void __launch_bounds__(64)
