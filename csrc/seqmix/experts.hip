@@ -1,0 +1,275 @@
+// Mixture of experts: the router with a group-limited choice, the expert matrix products over
+// the routed rows, and the weighted sum of the chosen experts' outputs.
+//
+// group_route_k: z = h . Wr^T in fp32, s = sigmoid(z).  The E experts form `groups` equal groups
+// of neighbours; a group's score is the sum of its two largest s; only experts of the best
+// `keep` groups can be chosen, and among them the `top` largest s win (ties: the lower index).
+// The weights are the chosen s as they are.  A token r routed to its k-th expert is slot
+// r * top + k; every expert gets the list of its slots (cnt / rows).
+//
+// expert_gemm: for expert e and each of its slots s: out[s] = x[s / x_div] . W_e^T.  Rows are
+// gathered through the slot lists, so only experts with rows read their weights.  bf16 runs
+// on the matrix cores (operands straight from global memory into MFMA fragments: the A rows
+// are gathered anyway and the weights of an expert are shared through L2 by the blocks that
+// work on it); fp32 and odd shapes run a tiled FMA kernel.  A slot's result does not depend on
+// which other slots share its tile.
+#include "common.h"
+using namespace sm;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// best (value, index) over the wavefront; ties go to the lower index
+__device__ __forceinline__ void wave_argmax(float& v, int& i) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    float ov = __shfl_xor(v, o, 64);
+    int oi = __shfl_xor(i, o, 64);
+    if (ov > v || (ov == v && oi < i)) {
+      v = ov;
+      i = oi;
+    }
+  }
+}
+
+// orders one wavefront's LDS writes before its later reads by other lanes
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+group_route_k(const T* __restrict__ h, int ldh, const float* __restrict__ wr, int W, int E, int top,
+              int groups, int keep, int* __restrict__ ids, float* __restrict__ wts,
+              int* __restrict__ cnt, int* __restrict__ rows, int ldr) {
+  extern __shared__ float smem[];
+  float* sh = smem;          // [W] the row in fp32
+  float* ss = sh + W;        // [E] scores; -1 marks "cannot be chosen (any more)"
+  float* sgs = ss + E;       // [groups] group scores
+  const int r = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) sh[i] = ldf(h, (size_t)r * ldh + i);
+  __syncthreads();
+  for (int e = wave; e < E; e += nw) {
+    const float* w = wr + (size_t)e * W;
+    float d = 0.0f;
+    for (int i = lane; i < W; i += 64) d += sh[i] * w[i];
+    d = wave_sum(d);
+    if (lane == 0) ss[e] = sigmoidf_(d);
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  const int per = E / groups;
+  if (keep < groups) {
+    for (int g = lane; g < groups; g += 64) {
+      float b1 = -1.0f, b2 = -1.0f;   // the two largest of the group
+      for (int i = 0; i < per; i++) {
+        float v = ss[g * per + i];
+        if (v > b1) { b2 = b1; b1 = v; }
+        else if (v > b2) b2 = v;
+      }
+      sgs[g] = b1 + (per > 1 ? b2 : 0.0f);
+    }
+    wave_sync();
+    // keep the best groups: pick `keep` times, then strike out the experts of the others
+    for (int k = 0; k < keep; k++) {
+      float bv = -INFINITY;
+      int bi = 1 << 30;
+      for (int g = lane; g < groups; g += 64) {
+        float v = sgs[g];
+        if (v > bv) { bv = v; bi = g; }     // ascending g: the first of equals stays
+      }
+      wave_argmax(bv, bi);
+      if (lane == 0) sgs[bi] = -INFINITY;   // marks "kept"
+      wave_sync();
+    }
+    for (int e = lane; e < E; e += 64)
+      if (sgs[e / per] != -INFINITY) ss[e] = -1.0f;
+    wave_sync();
+  }
+  for (int k = 0; k < top; k++) {
+    float bv = -INFINITY;
+    int bi = 1 << 30;
+    for (int e = lane; e < E; e += 64) {
+      float v = ss[e];
+      if (v > bv) { bv = v; bi = e; }
+    }
+    wave_argmax(bv, bi);
+    if (lane == 0) {
+      ss[bi] = -2.0f;
+      int slot = r * top + k;
+      ids[slot] = bi;
+      wts[slot] = bv;
+      int at = atomicAdd(&cnt[bi], 1);
+      rows[(size_t)bi * ldr + at] = slot;
+    }
+    wave_sync();
+  }
+}
+
+// bf16 on the matrix cores: a block of 4 wavefronts takes 64 slots x 64 output columns of one
+// expert; wavefront w owns 16 slots and walks K in steps of 32 with one A fragment (its
+// gathered rows) and four B fragments (16 weight rows each) per step.
+__global__ void __launch_bounds__(256)
+expert_gemm_mfma_k(const bf16* __restrict__ x, int ldx, int x_div, const bf16* __restrict__ w,
+                   const int* __restrict__ cnt, const int* __restrict__ rows, int ldr,
+                   bf16* __restrict__ out, int ldo, int N, int K) {
+  const int e = blockIdx.z, c = cnt[e];
+  const int m0 = blockIdx.x * 64, n0 = blockIdx.y * 64;
+  if (m0 >= c) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n16 = lane & 15, quad = lane >> 4;
+  const int mi = m0 + wave * 16 + n16;
+  const int slot = mi < c ? rows[(size_t)e * ldr + mi] : -1;
+  if (m0 + wave * 16 >= c) return;
+  const bf16* xa = slot >= 0 ? x + (size_t)(slot / x_div) * ldx : nullptr;
+  const bf16* wb[4];
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    int n = n0 + t * 16 + n16;
+    wb[t] = n < N ? w + ((size_t)e * N + n) * K : nullptr;
+  }
+  f32x4 acc[4];
+#pragma unroll
+  for (int t = 0; t < 4; t++) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    int kc = k0 + quad * 8;
+    bool kin = kc < K;                       // K is a multiple of 8
+    uint4 av = (xa && kin) ? *(const uint4*)(xa + kc) : make_uint4(0, 0, 0, 0);
+    uint4 bv[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+      bv[t] = (wb[t] && kin) ? *(const uint4*)(wb[t] + kc) : make_uint4(0, 0, 0, 0);
+    bf16x8 af = __builtin_bit_cast(bf16x8, av);
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, __builtin_bit_cast(bf16x8, bv[t]),
+                                                        acc[t], 0, 0, 0);
+  }
+  // accumulator layout: row quad*4 + i of the wave's 16 slots, column n16 of each tile
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    int so = __shfl(slot, quad * 4 + i, 64);
+    if (so < 0) continue;
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      int n = n0 + t * 16 + n16;
+      if (n < N) out[(size_t)so * ldo + n] = __float2bfloat16(acc[t][i]);
+    }
+  }
+}
+
+// any type, any shape: 32 slots x 64 columns per block, K staged through LDS 32 at a time
+#define EG_KT 32
+template <typename T>
+__global__ void __launch_bounds__(256)
+expert_gemm_fma_k(const T* __restrict__ x, int ldx, int x_div, const T* __restrict__ w,
+                  const int* __restrict__ cnt, const int* __restrict__ rows, int ldr,
+                  T* __restrict__ out, int ldo, int N, int K) {
+  __shared__ float sx[32][EG_KT + 1];
+  __shared__ float sw[64][EG_KT + 1];
+  __shared__ int sslot[32];
+  const int e = blockIdx.z, c = cnt[e];
+  const int m0 = blockIdx.x * 32, n0 = blockIdx.y * 64;
+  if (m0 >= c) return;
+  const int tid = threadIdx.x;
+  if (tid < 32) sslot[tid] = m0 + tid < c ? rows[(size_t)e * ldr + m0 + tid] : -1;
+  __syncthreads();
+  // thread (ty, tx): slots ty*2 .. ty*2+1, columns tx + 16*u
+  const int tx = tid & 15, ty = tid >> 4;
+  float acc[2][4];
+#pragma unroll
+  for (int a = 0; a < 2; a++)
+#pragma unroll
+    for (int u = 0; u < 4; u++) acc[a][u] = 0.0f;
+  for (int k0 = 0; k0 < K; k0 += EG_KT) {
+    for (int idx = tid; idx < 32 * EG_KT; idx += 256) {
+      int m = idx / EG_KT, k = idx % EG_KT;
+      int s = sslot[m];
+      sx[m][k] = (s >= 0 && k0 + k < K) ? ldf(x, (size_t)(s / x_div) * ldx + k0 + k) : 0.0f;
+    }
+    for (int idx = tid; idx < 64 * EG_KT; idx += 256) {
+      int n = idx / EG_KT, k = idx % EG_KT;
+      sw[n][k] = (n0 + n < N && k0 + k < K) ? ldf(w, ((size_t)e * N + n0 + n) * K + k0 + k) : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int k = 0; k < EG_KT; k++) {
+      float xa = sx[ty * 2][k], xb = sx[ty * 2 + 1][k];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        float wv = sw[tx + 16 * u][k];
+        acc[0][u] += xa * wv;
+        acc[1][u] += xb * wv;
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int a = 0; a < 2; a++) {
+    int s = sslot[ty * 2 + a];
+    if (s < 0) continue;
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      int n = n0 + tx + 16 * u;
+      if (n < N) stf(out, (size_t)s * ldo + n, acc[a][u]);
+    }
+  }
+}
+
+template <typename T>
+__global__ void expert_combine_k(const T* __restrict__ y, int ldy, const float* __restrict__ wts,
+                                 T* __restrict__ out, int ldo, int top, int n) {
+  int c = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y;
+  if (c >= n) return;
+  float s = 0.0f;
+  for (int k = 0; k < top; k++) s += wts[r * top + k] * ldf(y, (size_t)(r * top + k) * ldy + c);
+  stf(out, (size_t)r * ldo + c, s);
+}
+
+extern "C" {
+
+// cnt must be zero on entry
+int p2p_sm_group_route(const void* h, int ldh, const float* wr, int R, int W, int E, int top,
+                       int groups, int keep, int* ids, float* wts, int* cnt, int* rows, int ldr,
+                       int f32, hipStream_t st) {
+  if (R <= 0) return 0;
+  if (E < 1 || groups < 1 || E % groups || keep < 1 || keep > groups || top < 1 ||
+      top > keep * (E / groups) || ldr < R * top)
+    return (int)hipErrorInvalidValue;
+  size_t shm = (size_t)(W + E + groups) * 4;
+  if (shm > 64 * 1024) return (int)hipErrorInvalidValue;
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(group_route_k<T>, dim3(R), dim3(256), shm, st,
+                                         (const T*)h, ldh, wr, W, E, top, groups, keep, ids, wts,
+                                         cnt, rows, ldr));
+  return (int)hipGetLastError();
+}
+
+// max_slots: the most slots any expert can hold (the grid covers that many)
+int p2p_sm_expert_gemm(const void* x, int ldx, int x_div, const void* w, const int* cnt,
+                       const int* rows, int ldr, void* out, int ldo, int E, int N, int K,
+                       int max_slots, int f32, hipStream_t st) {
+  if (max_slots <= 0 || E <= 0) return 0;
+  if (x_div < 1 || N < 1 || K < 1) return (int)hipErrorInvalidValue;
+  if (!f32 && K % 8 == 0 && ldx % 8 == 0 && ((size_t)x & 15) == 0 && ((size_t)w & 15) == 0) {
+    dim3 grid((max_slots + 63) / 64, (N + 63) / 64, E);
+    hipLaunchKernelGGL(expert_gemm_mfma_k, grid, dim3(256), 0, st, (const bf16*)x, ldx, x_div,
+                       (const bf16*)w, cnt, rows, ldr, (bf16*)out, ldo, N, K);
+    return (int)hipGetLastError();
+  }
+  dim3 grid((max_slots + 31) / 32, (N + 63) / 64, E);
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(expert_gemm_fma_k<T>, grid, dim3(256), 0, st,
+                                         (const T*)x, ldx, x_div, (const T*)w, cnt, rows, ldr,
+                                         (T*)out, ldo, N, K));
+  return (int)hipGetLastError();
+}
+
+int p2p_sm_expert_combine(const void* y, int ldy, const float* wts, void* out, int ldo, int R,
+                          int top, int n, int f32, hipStream_t st) {
+  if (R <= 0) return 0;
+  dim3 g((n + 255) / 256, R), b(256);
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(expert_combine_k<T>, g, b, 0, st, (const T*)y, ldy, wts,
+                                         (T*)out, ldo, top, n));
+  return (int)hipGetLastError();
+}
+
+}  // extern "C"

@@ -1,6 +1,7 @@
 // Embedding with learned positions, RMS norms over fp32 or activation-typed rows (whole
-// row or equal parts, optional scatter of the rows), and the post-sublayer
-// norm + layer scale + residual add on the fp32 residual stream.
+// row or equal parts, optional scatter of the rows), and the post-sublayer passes on the fp32
+// residual stream: norm + layer scale + residual add, and the gated form
+// x += N(y * sigmoid(g + b)) * w with the norm N taken over equal parts of the row.
 #include "common.h"
 using namespace sm;
 
@@ -133,7 +134,95 @@ __global__ void norm_scale_add_k(float* __restrict__ x, const T* __restrict__ y,
     stf(h, (size_t)r * ldh + i, xr[i] * r2 * w2[i]);
 }
 
+// out[r] = embed[ids[r]] as fp32, and (optionally) the same row in the activation type
+template <typename T>
+__global__ void embed_rows_k(const T* __restrict__ embed, const int* __restrict__ ids,
+                             float* __restrict__ out, T* __restrict__ h, int ldh, int W) {
+  int r = blockIdx.x;
+  size_t eo = (size_t)ids[r] * W;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float v = ldf(embed, eo + i);
+    out[(size_t)r * W + i] = v;
+    if (h) stf(h, (size_t)r * ldh + i, v);
+  }
+}
+
+// one block per (row, part): x += v / sqrt(mean(v^2) + eps) * w with v = y * sigmoid(g + gb),
+// the mean over the part; h (optional) receives the updated residual in the activation type
+template <typename T>
+__global__ void gate_norm_add_k(float* __restrict__ x, const T* __restrict__ y, int ldy,
+                                const T* __restrict__ g, int ldg, const float* __restrict__ gb,
+                                const float* __restrict__ w, int n, int parts, float eps,
+                                T* __restrict__ h, int ldh) {
+  __shared__ float red[16];
+  int r = blockIdx.x / parts, p = blockIdx.x % parts;
+  int np = n / parts, c0 = p * np;
+  const T* yr = y + (size_t)r * ldy + c0;
+  const T* gr = g + (size_t)r * ldg + c0;
+  float* xr = x + (size_t)r * n + c0;
+  if (np <= NV * (int)blockDim.x) {
+    float v[NV], wv[NV], xv[NV];
+    float ss = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+      int i = threadIdx.x + k * blockDim.x;
+      bool ok = i < np;
+      float yv = ok ? ldf(yr, i) : 0.0f;
+      float gv = ok ? ldf(gr, i) + gb[c0 + i] : 0.0f;
+      wv[k] = ok ? w[c0 + i] : 0.0f;
+      xv[k] = ok ? xr[i] : 0.0f;
+      v[k] = yv * sigmoidf_(gv);
+      ss += v[k] * v[k];
+    }
+    ss = block_sum(ss, red);
+    float rs = 1.0f / sqrtf(ss / (float)np + eps);
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+      int i = threadIdx.x + k * blockDim.x;
+      if (i < np) {
+        float nv = xv[k] + v[k] * rs * wv[k];
+        xr[i] = nv;
+        if (h) stf(h, (size_t)r * ldh + c0 + i, nv);
+      }
+    }
+    return;
+  }
+  float ss = 0.0f;
+  for (int i = threadIdx.x; i < np; i += blockDim.x) {
+    float v = ldf(yr, i) * sigmoidf_(ldf(gr, i) + gb[c0 + i]);
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  float rs = 1.0f / sqrtf(ss / (float)np + eps);
+  for (int i = threadIdx.x; i < np; i += blockDim.x) {
+    float v = ldf(yr, i) * sigmoidf_(ldf(gr, i) + gb[c0 + i]);
+    float nv = xr[i] + v * rs * w[c0 + i];
+    xr[i] = nv;
+    if (h) stf(h, (size_t)r * ldh + c0 + i, nv);
+  }
+}
+
 extern "C" {
+
+int p2p_sm_embed_rows(const void* embed, const int* ids, float* out, void* h, int ldh, int R,
+                      int W, int f32, hipStream_t st) {
+  if (R <= 0) return 0;
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(embed_rows_k<T>, dim3(R), dim3(256), 0, st,
+                                         (const T*)embed, ids, out, (T*)h, ldh, W));
+  return (int)hipGetLastError();
+}
+
+// h (optional) has the activation type of y and g
+int p2p_sm_gate_norm_add(float* x, const void* y, int ldy, const void* g, int ldg,
+                         const float* gb, const float* w, int R, int n, int parts, float eps,
+                         void* h, int ldh, int h_f32, int f32, hipStream_t st) {
+  if (R <= 0) return 0;
+  if (parts <= 0 || n % parts || (h && h_f32 != f32)) return (int)hipErrorInvalidValue;
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(gate_norm_add_k<T>, dim3(R * parts), dim3(256), 0, st, x,
+                                         (const T*)y, ldy, (const T*)g, ldg, gb, w, n, parts, eps,
+                                         (T*)h, ldh));
+  return (int)hipGetLastError();
+}
 
 int p2p_sm_embed_pos(const void* embed, const void* ptab, const int* ids, const int* pos,
                      float* out, int R, int W, int f32, hipStream_t st) {

@@ -1,6 +1,7 @@
 // Pointwise pieces between the matrix products: tanh in place, sigmoid output gates with
-// arbitrary input strides, and the clamped gated feed-forward activation
-//   g = min(gate, limit), u = clamp(up, -limit, limit), y = g * sigmoid(1.702 g) * (u + 1).
+// arbitrary input strides, the clamped gated feed-forward activation
+//   g = min(gate, limit), u = clamp(up, -limit, limit), y = g * sigmoid(1.702 g) * (u + 1),
+// the silu-gated one, silu(gate) * up, and the tanh cap of the logits.
 #include "common.h"
 using namespace sm;
 
@@ -31,7 +32,38 @@ __global__ void ff_act_k(const T* __restrict__ gu, int ld, T* __restrict__ out, 
   stf(out, (size_t)r * ldo + c, g * sigmoidf_(alpha * g) * (u + 1.0f));
 }
 
+template <typename T>
+__global__ void glu_act_k(const T* __restrict__ gu, int ld, T* __restrict__ out, int ldo, int F) {
+  int c = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y;
+  if (c >= F) return;
+  float g = ldf(gu, (size_t)r * ld + c);
+  stf(out, (size_t)r * ldo + c, g * sigmoidf_(g) * ldf(gu, (size_t)r * ld + F + c));
+}
+
+template <typename T>
+__global__ void softcap_k(const T* __restrict__ y, int ld, float* __restrict__ out, int n,
+                          float cap) {
+  int c = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y;
+  if (c < n) out[(size_t)r * n + c] = cap * tanhf(ldf(y, (size_t)r * ld + c) / cap);
+}
+
 extern "C" {
+
+int p2p_sm_glu_act(const void* gu, int ld, void* out, int ldo, int R, int F, int f32,
+                   hipStream_t st) {
+  if (R <= 0) return 0;
+  dim3 g((F + 255) / 256, R), b(256);
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(glu_act_k<T>, g, b, 0, st, (const T*)gu, ld, (T*)out, ldo, F));
+  return (int)hipGetLastError();
+}
+
+int p2p_sm_softcap(const void* y, int ld, float* out, int R, int n, float cap, int f32,
+                   hipStream_t st) {
+  if (R <= 0 || n <= 0) return 0;
+  dim3 g((n + 255) / 256, R), b(256);
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(softcap_k<T>, g, b, 0, st, (const T*)y, ld, out, n, cap));
+  return (int)hipGetLastError();
+}
 
 int p2p_sm_tanh(void* x, int ld, int n, int R, int f32, hipStream_t st) {
   if (R <= 0 || n <= 0) return 0;

@@ -1,0 +1,213 @@
+// Grouped-query attention over a paged key/value pool: the pass that prepares its inputs and
+// the attention kernel in fp32 arithmetic (float32 models, shapes the matrix-core kernel does
+// not take).
+//
+// qk_norm_rope_store_k: one projection buffer holds q (H heads x D) | k (G x D) | v (G x V) of a
+// row.  q and k are RMS-normalised over their whole rows (all heads at once), weighted, and the
+// channel pairs (2i, 2i+1), i < nrot, of every head are turned by the angle pos * inv_freq[i]:
+// (a, b) -> (a cos - b sin, b cos + a sin).  q goes to its own buffer, k | v to the row of the
+// paged pool that the token owns.  Norm, angle and rotation are fp32.
+//
+// window_attn_k: pool row = [k of G heads | v of G heads]; query head h reads key/value head
+// h / (H/G).  Causal sliding window: position i sees j with 0 <= i - j < win.  The softmax
+// denominator holds one more term exp(sink_h) with no key and no value: the running maximum
+// starts at sink_h and the running sum at 1.  One block per (query row, key/value head): the
+// heads of the group share the key and value tiles, which stream through LDS with an online
+// softmax.
+#include "common.h"
+using namespace sm;
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_store_k(const T* __restrict__ proj, int ldp, int H, int G, int D, int V,
+                     const float* __restrict__ qw, const float* __restrict__ kw,
+                     const float* __restrict__ inv_freq, int nrot, const int* __restrict__ pos,
+                     const int* __restrict__ cache_rows, T* __restrict__ pool, float eps,
+                     T* __restrict__ q_out, int ldq) {
+  __shared__ float red[16];
+  const int r = blockIdx.x;
+  const int nq = H * D, nk = G * D, nv = G * V;
+  const T* row = proj + (size_t)r * ldp;
+  float sq = 0.0f, sk = 0.0f;
+  for (int i = threadIdx.x; i < nq; i += blockDim.x) {
+    float v = ldf(row, i);
+    sq += v * v;
+  }
+  for (int i = threadIdx.x; i < nk; i += blockDim.x) {
+    float v = ldf(row, nq + i);
+    sk += v * v;
+  }
+  sq = block_sum(sq, red);
+  sk = block_sum(sk, red);
+  const float rq = 1.0f / sqrtf(sq / (float)nq + eps), rk = 1.0f / sqrtf(sk / (float)nk + eps);
+  const float p = (float)pos[r];
+  const int D2 = (D + 1) / 2;
+  T* crow = pool + (size_t)cache_rows[r] * (nk + nv);
+  T* qrow = q_out + (size_t)r * ldq;
+  // pairs of q, then pairs of k
+  for (int idx = threadIdx.x; idx < (H + G) * D2; idx += blockDim.x) {
+    int hh = idx / D2, j = idx % D2;
+    bool isq = hh < H;
+    int c = (isq ? hh : hh - H) * D + 2 * j;        // channel within q or k
+    bool two = 2 * j + 1 < D;
+    const float* w = isq ? qw : kw;
+    float rs = isq ? rq : rk;
+    int off = isq ? 0 : nq;
+    float a = ldf(row, off + c) * rs * w[c];
+    float b = two ? ldf(row, off + c + 1) * rs * w[c + 1] : 0.0f;
+    if (j < nrot) {
+      float sn, cs;
+      sincosf(p * inv_freq[j], &sn, &cs);
+      float a2 = a * cs - b * sn, b2 = b * cs + a * sn;
+      a = a2;
+      b = b2;
+    }
+    T* dst = isq ? qrow : crow;
+    stf(dst, c, a);
+    if (two) stf(dst, c + 1, b);
+  }
+  for (int i = threadIdx.x; i < nv; i += blockDim.x) crow[nk + i] = row[nq + nk + i];
+}
+
+#define WA_TK 32       // keys per tile at most
+#define WA_THREADS 256
+#define WA_ACC 16      // (head, value channel) pairs per thread at most
+
+template <typename T>
+__global__ void __launch_bounds__(WA_THREADS)
+window_attn_k(const T* __restrict__ q, int ldq, const T* __restrict__ pool,
+              const int* __restrict__ bt, int max_pages, const int* __restrict__ row_ent,
+              const int* __restrict__ pos, const float* __restrict__ sink, float scale, int win,
+              T* __restrict__ out, int ldo, int H, int G, int D, int V, int page, int TK,
+              float out_scale) {
+  extern __shared__ float smem[];
+  const int HG = H / G, g = blockIdx.y, h0 = g * HG;
+  const int ldk = D + 1, ldv = V + 1, ldpool = G * (D + V);
+  float* sq = smem;                      // [HG][D]
+  float* sk = sq + HG * D;               // [TK][D + 1]
+  float* sv = sk + TK * ldk;             // [TK][V + 1]
+  float* sp = sv + TK * ldv;             // [HG][TK]
+  float* sm_ = sp + HG * TK;             // [HG] running max
+  float* sl = sm_ + HG;                  // [HG] running sum
+  float* sal = sl + HG;                  // [HG] rescale of this tile
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const int p = pos[r];
+  const int* pages = bt + (size_t)row_ent[r] * max_pages;
+  const int j_lo = max(0, p - win + 1);
+  for (int idx = tid; idx < HG * D; idx += WA_THREADS)
+    sq[idx] = ldf(q, (size_t)r * ldq + (size_t)h0 * D + idx);
+  if (tid < HG) {
+    sm_[tid] = sink[h0 + tid];
+    sl[tid] = 1.0f;
+  }
+  float acc[WA_ACC];
+#pragma unroll
+  for (int a = 0; a < WA_ACC; a++) acc[a] = 0.0f;
+  const int npair = HG * V;
+  for (int j0 = j_lo; j0 <= p; j0 += TK) {
+    int nk = min(TK, p + 1 - j0);
+    __syncthreads();  // previous tile fully consumed (and sq / sm_ / sl initialised)
+    for (int idx = tid; idx < nk * D; idx += WA_THREADS) {
+      int jj = idx / D, c = idx % D;
+      int j = j0 + jj;
+      size_t tok = (size_t)pages[j / page] * page + (j % page);
+      sk[jj * ldk + c] = ldf(pool, tok * ldpool + (size_t)g * D + c);
+    }
+    for (int idx = tid; idx < nk * V; idx += WA_THREADS) {
+      int jj = idx / V, c = idx % V;
+      int j = j0 + jj;
+      size_t tok = (size_t)pages[j / page] * page + (j % page);
+      sv[jj * ldv + c] = ldf(pool, tok * ldpool + (size_t)G * D + (size_t)g * V + c);
+    }
+    __syncthreads();
+    for (int idx = tid; idx < HG * TK; idx += WA_THREADS) {
+      int h = idx / TK, jj = idx % TK;
+      float s = -INFINITY;
+      if (jj < nk) {
+        const float* qh = sq + h * D;
+        const float* kr = sk + jj * ldk;
+        float d = 0.0f;
+        for (int i = 0; i < D; i++) d += qh[i] * kr[i];
+        s = d * scale;
+      }
+      sp[idx] = s;
+    }
+    __syncthreads();
+    if (tid < HG) {
+      float mt = sm_[tid];
+      float mo = mt;
+      for (int jj = 0; jj < nk; jj++) mt = fmaxf(mt, sp[tid * TK + jj]);
+      sal[tid] = expf(mo - mt);
+      sm_[tid] = mt;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < HG * TK; idx += WA_THREADS) {
+      int h = idx / TK, jj = idx % TK;
+      sp[idx] = jj < nk ? expf(sp[idx] - sm_[h]) : 0.0f;
+    }
+    __syncthreads();
+    if (tid < HG) {
+      float l = sl[tid] * sal[tid];
+      for (int jj = 0; jj < nk; jj++) l += sp[tid * TK + jj];
+      sl[tid] = l;
+    }
+#pragma unroll
+    for (int a = 0; a < WA_ACC; a++) {
+      int idx = tid + a * WA_THREADS;
+      if (idx < npair) {
+        int h = idx / V, c = idx % V;
+        float v = acc[a] * sal[h];
+        const float* pr = sp + h * TK;
+        for (int jj = 0; jj < nk; jj++) v += pr[jj] * sv[jj * ldv + c];
+        acc[a] = v;
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int a = 0; a < WA_ACC; a++) {
+    int idx = tid + a * WA_THREADS;
+    if (idx < npair) {
+      int h = idx / V;
+      stf(out, (size_t)r * ldo + (size_t)h0 * V + idx, acc[a] / sl[h] * out_scale);
+    }
+  }
+}
+
+extern "C" {
+
+int p2p_sm_qk_norm_rope_store(const void* proj, int ldp, int H, int G, int D, int V,
+                              const float* qw, const float* kw, const float* inv_freq, int nrot,
+                              const int* pos, const int* cache_rows, void* pool, float eps,
+                              void* q_out, int ldq, int R, int f32, hipStream_t st) {
+  if (R <= 0) return 0;
+  if (H < 1 || G < 1 || D < 1 || V < 1 || nrot < 0 || 2 * nrot > D) return (int)hipErrorInvalidValue;
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(qk_norm_rope_store_k<T>, dim3(R), dim3(256), 0, st,
+                                         (const T*)proj, ldp, H, G, D, V, qw, kw, inv_freq, nrot,
+                                         pos, cache_rows, (T*)pool, eps, (T*)q_out, ldq));
+  return (int)hipGetLastError();
+}
+
+int p2p_sm_window_attn(const void* q, int ldq, const void* pool, const int* bt, int max_pages,
+                       const int* row_ent, const int* pos, const float* sink, float scale, int win,
+                       void* out, int ldo, int R, int H, int G, int D, int V, int page,
+                       float out_scale, int f32, hipStream_t st) {
+  if (R <= 0) return 0;
+  if (H < 1 || G < 1 || H % G || D < 1 || V < 1 || win < 1) return (int)hipErrorInvalidValue;
+  int HG = H / G, TK = WA_TK;
+  auto lds = [&](int tk) {
+    return ((size_t)HG * D + (size_t)tk * (D + 1) + (size_t)tk * (V + 1) + (size_t)HG * tk +
+            3 * HG) * 4;
+  };
+  while (TK > 2 && lds(TK) > 64 * 1024) TK /= 2;
+  if ((long)HG * V > (long)WA_ACC * WA_THREADS || HG > WA_THREADS || lds(TK) > 64 * 1024)
+    return (int)hipErrorInvalidValue;
+  dim3 grid(R, G);
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(window_attn_k<T>, grid, dim3(WA_THREADS), lds(TK), st,
+                                         (const T*)q, ldq, (const T*)pool, bt, max_pages, row_ent,
+                                         pos, sink, scale, win, (T*)out, ldo, H, G, D, V, page, TK,
+                                         out_scale));
+  return (int)hipGetLastError();
+}
+
+}  // extern "C"

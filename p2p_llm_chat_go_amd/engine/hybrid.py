@@ -22,7 +22,7 @@ import torch
 from ..models.hybrid import HybridConfig, HybridModel, HybridWeights, StepBatch
 from ..ops import PAGE
 from .engine import GenResult
-from .seq_cache import SequenceCache
+from .seq_cache import SequenceCache, layer_specs
 
 
 DECODE_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
@@ -98,7 +98,7 @@ class HybridEngine:
         slots = num_slots or max_batch
         specs = weights.cache_specs()
         if kv_pages is None:
-            per_page = max(1, sum(int(s[1]) for s in specs if s and s[0] == "paged")
+            per_page = max(1, sum(int(what) for _i, kind, what in layer_specs(specs) if kind == "paged")
                            * PAGE * (4 if self.dtype == torch.float32 else 2))
             if self.device.type == "cuda":
                 free, _ = torch.cuda.mem_get_info(self.device)

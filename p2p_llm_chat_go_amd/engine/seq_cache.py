@@ -1,7 +1,8 @@
 """Sequence cache of hybrid models: a paged pool for what attention layers keep per token
 and fixed state slots for what recurrent layers carry per sequence.
 
-Every layer declares what it needs (``Mixer.cache_spec``):
+Every layer declares what it needs (``Mixer.cache_spec``; a mixer made of several gives a
+list):
   * ``("paged", width)``  -- one vector of ``width`` numbers per token, stored in pages of
     ``PAGE`` tokens drawn from the shared ``PageAllocator`` (page 0 is the null page); a
     sequence's token t lives at ``pages[t // PAGE] * PAGE + t % PAGE`` in every paged layer;
@@ -17,6 +18,16 @@ import torch
 
 from ..ops import PAGE
 from .kv_cache import PageAllocator, pages_for
+
+
+def layer_specs(specs: list):
+    """(layer, kind, what) for every declaration; a layer may give one spec, a list of specs
+    (a mixer made of several) or None."""
+    for i, spec in enumerate(specs):
+        if not spec:
+            continue
+        for kind, what in (spec if isinstance(spec, list) else [spec]):
+            yield i, kind, what
 
 
 class SlotAllocator:
@@ -56,18 +67,21 @@ class SequenceCache:
         self.allocator = PageAllocator(num_pages)
         self.slots = SlotAllocator(num_slots)
         self.paged, self.state = {}, {}
-        for i, spec in enumerate(specs):
-            if spec is None:
-                continue
-            kind, what = spec
+        for i, kind, what in layer_specs(specs):
             if kind == "paged":
+                if i in self.paged:
+                    raise ValueError("layer %d declares two paged pools" % i)
                 self.paged[i] = torch.zeros(num_pages * PAGE, int(what), device=self.device,
                                             dtype=dtype)
             elif kind == "state":
                 # one slot more than the allocator hands out: the null slot, where padding rows
                 # of a bucketed (graph-captured) step keep their state, like the null page
-                self.state[i] = {k: torch.zeros((num_slots + 1,) + tuple(s), device=self.device,
-                                                dtype=torch.float32) for k, s in what.items()}
+                st = self.state.setdefault(i, {})
+                for k, s in what.items():
+                    if k in st:
+                        raise ValueError("layer %d declares state %r twice" % (i, k))
+                    st[k] = torch.zeros((num_slots + 1,) + tuple(s), device=self.device,
+                                        dtype=torch.float32)
             else:
                 raise ValueError("unknown cache kind %r" % kind)
         self.null_slot = num_slots

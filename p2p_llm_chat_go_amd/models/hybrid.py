@@ -1,21 +1,37 @@
 """Hybrid decoders: a configurable stack of sequence mixers on an fp32 residual stream.
 
 A model is a list of layers; each layer has one *mixer* (registered in ``MIXERS``) and
-optionally a feed-forward, both wrapped as
+optionally a feed-forward (``FEEDFORWARDS``).  A design (``DESIGNS``) fixes how a sublayer f
+is wrapped around the residual stream,
 
-    x <- x + scale * norm_b(sublayer(norm_a(x)))        (RMS norms, per-channel layer scale)
+    "sandwich"    x <- x + scale * norm_b(f(norm_a(x)))      RMS norms, per-channel layer scale
+    "gated_post"  x <- x + norm(f(x) * sigmoid(R x + b))     the sublayer reads x itself; the
+                                                             norm is taken in equal parts
 
-with learned absolute positions added to the token embedding.  Mixers:
+and whether learned absolute positions are added to the token embedding.  Mixers:
 
   ``general_delta``     generalized delta rule: per head a D x D state with per-channel decay
                         and an in-context removal of the unit key direction;
   ``mamba2``            Mamba-2 selective state space (short causal convolution + scan);
   ``latent_attention``  attention over a cached low-rank latent per token (keys and values
                         are up-projections of it), causal sliding window, softmax with a
-                        learned per-head sink, sigmoid output gate, no positional rotation.
+                        learned per-head sink, sigmoid output gate, no positional rotation;
+  ``window_attention``  grouped-query attention over cached keys and values: RMS norm of the
+                        whole query / key projection, interleaved rotary positions on the
+                        first channels of each head, causal sliding window, softmax sink;
+  ``gated_delta``       gated delta rule: short causal convolutions + silu on q, k, v, unit
+                        keys, a per-channel decay and a write that corrects what the key reads;
+  ``hgrn2``             linear attention whose forget gate also sets what is written;
+  ``parallel``          two mixers side by side on the same input, summed with fixed scales.
 
-"Regesun" is the design that stacks these three; its checkpoints are a ``config.json`` with
-``architecture: "Regesun"`` and one safetensors file (``load_dir``).
+Feed-forwards: ``dense`` (silu-gated, or the clamped gated unit when the config gives a
+limit) and ``moe`` (sigmoid router, choice limited to the best groups of experts).
+
+"Regesun" stacks the first three mixers in the sandwich form with learned positions;
+"Rotutar" stacks ``parallel`` (window attention beside the gated delta rule) and ``hgrn2``
+layers in the gated post-norm form, without positions other than the rotation, and caps
+its logits with a tanh.  A checkpoint is a ``config.json`` whose ``architecture`` names the
+design and one safetensors file (``load_dir``).
 
 One ``forward`` serves every step: a flat list of token rows cut into entries (portions of
 prompts and single decoded tokens side by side, ``StepBatch``); attention layers read and
@@ -47,6 +63,16 @@ class LayerSpec:
 
 
 @dataclasses.dataclass(frozen=True)
+class Design:
+    block: str                # how sublayers sit on the residual stream: "sandwich" | "gated_post"
+    positions: str | None     # "learned": a position table is added to the embedding
+
+
+DESIGNS = {"Regesun": Design("sandwich", "learned"), "Rotutar": Design("gated_post", None)}
+NO_POS_LIMIT = 1 << 30
+
+
+@dataclasses.dataclass(frozen=True)
 class HybridConfig:
     name: str
     width: int
@@ -57,6 +83,13 @@ class HybridConfig:
     bos_id: int = 1
     eos_ids: tuple = ()
     is_moe: bool = False
+    design: str = "Regesun"
+    norm_groups: int = 1
+    logit_softcap: float = 0.0
+
+    @property
+    def traits(self) -> Design:
+        return DESIGNS[self.design]
 
     @property
     def n_layers(self) -> int:
@@ -70,34 +103,46 @@ class HybridConfig:
     def from_dict(cls, c: dict, name: str | None = None) -> "HybridConfig":
         layers = tuple(LayerSpec(L["type"], dict(L["mixer"]), dict(L["mlp"]) if L.get("mlp") else None)
                        for L in c["layers"])
+        design = str(c.get("architecture", "Regesun"))
+        if design not in DESIGNS:
+            raise KeyError("unknown design %r (known: %s)" % (design, ", ".join(sorted(DESIGNS))))
         for L in layers:
             if L.kind not in MIXERS:
                 raise KeyError("unknown mixer %r (known: %s)" % (L.kind, ", ".join(sorted(MIXERS))))
-            if L.mlp is not None and L.mlp.get("kind", "dense") != "dense":
+            if L.mlp is not None and L.mlp.get("kind", "dense") not in FEEDFORWARDS:
                 raise KeyError("unknown feed-forward kind %r" % L.mlp.get("kind"))
         eos = c.get("eos_token_id", ())
         eos = tuple(eos) if isinstance(eos, (list, tuple)) else (int(eos),)
-        return cls(name=name or str(c.get("architecture", "hybrid")).lower(), width=int(c["width"]),
+        width, groups = int(c["width"]), int(c["norm"].get("groups", 1))
+        if groups < 1 or width % groups:
+            raise ValueError("width %d does not split into %d norm groups" % (width, groups))
+        max_pos = int(c["max_positions"]) if DESIGNS[design].positions else \
+            int(c.get("max_positions", NO_POS_LIMIT))
+        return cls(name=name or design.lower(), width=width,
                    vocab=int(c["vocab"]), layers=layers, eps=float(c["norm"]["eps"]),
-                   max_pos=int(c["max_positions"]), bos_id=int(c.get("bos_token_id", 1)),
-                   eos_ids=eos)
+                   max_pos=max_pos, bos_id=int(c.get("bos_token_id", 1)),
+                   eos_ids=eos, design=design, norm_groups=groups,
+                   logit_softcap=float(c.get("logit_softcap") or 0.0),
+                   is_moe=any(L.mlp is not None and L.mlp.get("kind") == "moe" for L in layers))
 
     def resolve(self, shapes: dict) -> "HybridConfig":
-        """Fill the sizes that a config leaves to the checkpoint's tensor shapes (the rank of
-        the generalized delta rule's decay projection).  shapes: tensor name -> shape."""
+        """Fill the sizes that a config leaves to the checkpoint's tensor shapes (the ranks of
+        low-rank projections).  shapes: tensor name -> shape."""
         layers = []
         for i, L in enumerate(self.layers):
-            mx = dict(L.mixer)
-            k = "l%d.mix.w1" % i
-            if L.kind == "general_delta" and "decay_rank" not in mx and k in shapes:
-                mx["decay_rank"] = int(tuple(shapes[k])[0])
+            mx = MIXERS[L.kind].resolve_spec(dict(L.mixer), "l%d.mix." % i, shapes)
             layers.append(LayerSpec(L.kind, mx, L.mlp))
         return dataclasses.replace(self, layers=tuple(layers))
 
     def to_dict(self) -> dict:
-        return {"architecture": "Regesun", "width": self.width, "vocab": self.vocab,
-                "max_positions": self.max_pos, "norm": {"eps": self.eps},
-                "layers": [{"type": L.kind, "mixer": L.mixer, "mlp": L.mlp} for L in self.layers]}
+        d = {"architecture": self.design, "width": self.width, "vocab": self.vocab,
+             "norm": {"eps": self.eps, "groups": self.norm_groups},
+             "layers": [{"type": L.kind, "mixer": L.mixer, "mlp": L.mlp} for L in self.layers]}
+        if self.traits.positions or self.max_pos != NO_POS_LIMIT:
+            d["max_positions"] = self.max_pos
+        if self.logit_softcap:
+            d["logit_softcap"] = self.logit_softcap
+        return d
 
 
 def _vec(t, dev):
@@ -189,6 +234,11 @@ class Mixer:
     def __init__(self, spec: dict, width: int, eps: float):
         self.spec, self.width, self.eps = spec, width, eps
 
+    @staticmethod
+    def resolve_spec(spec: dict, prefix: str, shapes: dict) -> dict:
+        """Sizes that the checkpoint's tensor shapes give rather than the config."""
+        return spec
+
     def tensor_shapes(self) -> dict:
         raise NotImplementedError
 
@@ -196,15 +246,38 @@ class Mixer:
         raise NotImplementedError
 
     def cache_spec(self):
+        """("paged", width) | ("state", {name: shape}) | a list of those | None."""
         return None
 
-    def forward(self, h, b: StepBatch, cache, layer: int):
+    # A mixer either implements ``forward`` (it projects its input itself), or exposes the
+    # rows that read the layer input as ``w_in`` and implements ``mix`` on their product, so
+    # that whoever owns the input (a layer with a gate, a ``parallel`` mixer) can run every
+    # projection of the same input as one matrix product.
+    w_in = None
+    wo = None
+    n_mid = 0
+
+    def mix(self, proj, b: "StepBatch", cache, layer: int, out, out_scale: float = 1.0):
+        """proj [R, rows of w_in] -> out [R, n_mid] (the input of the output projection)."""
         raise NotImplementedError
+
+    def forward_proj(self, proj, b: "StepBatch", cache, layer: int):
+        mid = torch.empty(b.R, self.n_mid, device=proj.device, dtype=proj.dtype)
+        return F.linear(self.mix(proj, b, cache, layer, mid), self.wo)
+
+    def forward(self, h, b: "StepBatch", cache, layer: int):
+        return self.forward_proj(F.linear(h, self.w_in), b, cache, layer)
 
 
 class GeneralDelta(Mixer):
     kind = "general_delta"
     LOW_RANK = 32
+
+    @staticmethod
+    def resolve_spec(spec, prefix, shapes):
+        if "decay_rank" not in spec and prefix + "w1" in shapes:
+            spec["decay_rank"] = int(tuple(shapes[prefix + "w1"])[0])
+        return spec
 
     def tensor_shapes(self):
         n, W = self.spec["heads"] * self.spec["dim"], self.width
@@ -328,50 +401,320 @@ class LatentAttention(Mixer):
         return F.linear(gated, self.wo)
 
 
-MIXERS = {c.kind: c for c in (GeneralDelta, Mamba2, LatentAttention)}
+class WindowAttention(Mixer):
+    """Grouped-query attention with cached keys and values (``ops.seqmix.window_attn``)."""
+    kind = "window_attention"
+
+    def _dims(self):
+        s = self.spec
+        self.H, self.D, self.V = int(s["heads"]), int(s["dim"]), int(s["vdim"])
+        self.G = int(s.get("kv_heads", self.H))
+        self.win = int(s["mask"]["size"]) if s.get("mask") else 1 << 30
+        self.scale = float(s["scale"]) if "scale" in s else self.D ** -0.5
+        rot = s.get("rot")
+        self.rot_dims = int(rot["dims"]) if rot else 0
+        self.rot_base = float(rot["base"]) if rot else 1.0
+        if self.H % self.G or self.rot_dims % 2 or self.rot_dims > self.D:
+            raise ValueError("window_attention: %d heads / %d kv heads / %d rotated of %d channels"
+                             % (self.H, self.G, self.rot_dims, self.D))
+        self.n_mid = self.H * self.V
+
+    def tensor_shapes(self):
+        self._dims()
+        H, G, D, V, W = self.H, self.G, self.D, self.V, self.width
+        return {"q": (H * D, W), "k": (G * D, W), "v": (G * V, W), "q.norm": (H * D,),
+                "k.norm": (G * D,), "sink": (H,), "o": (W, H * V)}
+
+    def load(self, get, dtype, dev):
+        self._dims()
+        self.w_in = torch.cat([get("q"), get("k"), get("v")], 0).to(dev, dtype).contiguous()
+        self.qnorm, self.knorm, self.sink = (_vec(get(k), dev) for k in ("q.norm", "k.norm", "sink"))
+        self.inv_freq = sm.rope_inv_freq(self.rot_base, self.rot_dims, dev)
+        self.wo = get("o").to(dev, dtype).contiguous()
+
+    def cache_spec(self):
+        return ("paged", self.G * (self.D + self.V))
+
+    def mix(self, proj, b, cache, layer, out, out_scale=1.0):
+        H, G, D, V = self.H, self.G, self.D, self.V
+        pool = cache.paged[layer]
+        q = torch.empty(b.R, H * D, device=proj.device, dtype=proj.dtype)
+        sm.qk_norm_rope_store(proj, H, G, D, V, self.qnorm, self.knorm, self.inv_freq, b.pos,
+                              b.cache_rows, pool, self.eps, q)
+        units = b.units(sm.window_rows_per_wave(H // G)) if sm.window_mfma_ok(q, pool, D, V) else None
+        sm.window_attn(q, pool, b.block_tables, b.row_ent, b.pos, self.sink, self.scale, self.win,
+                       out, PAGE, H, G, D, V, units=units, max_keys=b.max_keys, out_scale=out_scale)
+        return out
+
+
+class GatedDelta(Mixer):
+    """Gated delta rule behind short convolutions (``ops.seqmix.gated_delta_scan``)."""
+    kind = "gated_delta"
+    LOW_RANK = 16
+
+    @staticmethod
+    def resolve_spec(spec, prefix, shapes):
+        for key, name in (("decay_rank", "a1"), ("gate_rank", "g1")):
+            if key not in spec and prefix + name in shapes:
+                spec[key] = int(tuple(shapes[prefix + name])[0])
+        return spec
+
+    def _dims(self):
+        s = self.spec
+        self.H, self.D, self.V, self.K = int(s["heads"]), int(s["dim"]), int(s["vdim"]), int(s["conv"])
+        self.G = int(s.get("kv_heads", self.H))
+        self.ra = int(s.get("decay_rank", self.LOW_RANK))
+        self.rg = int(s.get("gate_rank", self.LOW_RANK))
+        if self.H % self.G or self.K < 1:
+            raise ValueError("gated_delta: %d heads / %d kv heads / %d taps" % (self.H, self.G, self.K))
+        self.C = 2 * self.G * self.D + self.H * self.V
+        self.n_mid = self.H * self.V
+
+    def tensor_shapes(self):
+        self._dims()
+        H, G, D, V, K, W = self.H, self.G, self.D, self.V, self.K, self.width
+        return {"q": (G * D, W), "q.conv": (G * D, K), "k": (G * D, W), "k.conv": (G * D, K),
+                "v": (H * V, W), "v.conv": (H * V, K), "b": (H, W), "A_log": (H,), "norm": (V,),
+                "a1": (self.ra, W), "a2": (H * D, self.ra), "dt_bias": (H * D,),
+                "g1": (self.rg, W), "g2": (H * V, self.rg), "o": (W, H * V)}
+
+    def load(self, get, dtype, dev):
+        self._dims()
+        # one projection for everything that reads the layer input: q | k | v | beta | a1 | g1
+        self.w_in = torch.cat([get(k) for k in ("q", "k", "v", "b", "a1", "g1")], 0).to(dev, dtype).contiguous()
+        self.cw = torch.cat([_vec(get(k), dev) for k in ("q.conv", "k.conv", "v.conv")], 0).contiguous()
+        self.cb = torch.zeros(self.C, device=dev, dtype=torch.float32)
+        self.w_a2 = get("a2").to(dev, dtype).contiguous()
+        self.w_g2 = get("g2").to(dev, dtype).contiguous()
+        self.A_log, self.dt_bias, self.normw = (_vec(get(k), dev) for k in ("A_log", "dt_bias", "norm"))
+        self.wo = get("o").to(dev, dtype).contiguous()
+
+    def cache_spec(self):
+        return ("state", {"S": (self.H, self.D, self.V), "tail": (self.K - 1, self.C)})
+
+    def mix(self, proj, b, cache, layer, out, out_scale=1.0):
+        st, C, H = cache.state[layer], self.C, self.H
+        conv = torch.empty(b.R, C, device=proj.device, dtype=torch.float32)
+        sm.mamba_conv(proj, 0, self.cw, self.cb, st["tail"], b.ent, b.ent_host, b.row_ent, conv)
+        sm.conv_tail_roll(proj, 0, st["tail"], b.ent, b.ent_host, C)
+        araw = F.linear(proj[:, C + H:C + H + self.ra], self.w_a2)
+        gate = F.linear(proj[:, C + H + self.ra:C + H + self.ra + self.rg], self.w_g2)
+        sm.gated_delta_scan(conv, araw, proj[:, C:C + H], gate, self.A_log, self.dt_bias, self.normw,
+                            st["S"], b.ent, b.ent_host, out, H, self.G, self.D, self.V, self.eps,
+                            out_scale=out_scale)
+        return out
+
+
+class HGRN2(Mixer):
+    """Gated linear attention with a lower-bounded forget gate (``ops.seqmix.hgrn2_scan``)."""
+    kind = "hgrn2"
+
+    def _dims(self):
+        s = self.spec
+        self.H, self.D, self.V = int(s["heads"]), int(s["dim"]), int(s["vdim"])
+        self.n_mid = self.H * self.V
+
+    def tensor_shapes(self):
+        self._dims()
+        n, W = self.H * self.D, self.width
+        return {"q": (n, W), "f": (n, W), "f.b": (n,), "lower": (n,), "v": (self.H * self.V, W),
+                "norm": (self.V,), "o": (W, self.H * self.V)}
+
+    def load(self, get, dtype, dev):
+        self._dims()
+        self.w_in = torch.cat([get("q"), get("f"), get("v")], 0).to(dev, dtype).contiguous()
+        self.fb, self.lower, self.normw = (_vec(get(k), dev) for k in ("f.b", "lower", "norm"))
+        self.wo = get("o").to(dev, dtype).contiguous()
+
+    def cache_spec(self):
+        return ("state", {"S": (self.H, self.D, self.V)})
+
+    def mix(self, proj, b, cache, layer, out, out_scale=1.0):
+        sm.hgrn2_scan(proj, self.lower, self.fb, self.normw, cache.state[layer]["S"], b.ent,
+                      b.ent_host, out, self.H, self.D, self.V, self.eps, out_scale=out_scale)
+        return out
+
+
+class Parallel(Mixer):
+    """Two mixers on the same input: ``left_scale * left + right_scale * right``.  Their input
+    projections are one matrix product, and so are their output projections (each branch
+    writes its scaled share of one buffer)."""
+    kind = "parallel"
+    BRANCHES = (("left", "window_attention"), ("right", "gated_delta"))
+
+    def __init__(self, spec, width, eps):
+        super().__init__(spec, width, eps)
+        self.parts = [(name, MIXERS[spec[name].get("type", kind)](dict(spec[name]), width, eps),
+                       float(spec.get(name + "_scale", 1.0))) for name, kind in self.BRANCHES]
+
+    @staticmethod
+    def resolve_spec(spec, prefix, shapes):
+        for name, kind in Parallel.BRANCHES:
+            sub = dict(spec[name])
+            spec[name] = MIXERS[sub.get("type", kind)].resolve_spec(sub, prefix + name + ".", shapes)
+        return spec
+
+    def tensor_shapes(self):
+        return {name + "." + k: s for name, m, _ in self.parts for k, s in m.tensor_shapes().items()}
+
+    def load(self, get, dtype, dev):
+        for name, m, _ in self.parts:
+            m.load(lambda k, name=name: get(name + "." + k), dtype, dev)
+        self.w_in = torch.cat([m.w_in for _, m, _ in self.parts], 0).contiguous()
+        self.wo = torch.cat([m.wo for _, m, _ in self.parts], 1).contiguous()
+        self.n_mid = sum(m.n_mid for _, m, _ in self.parts)
+
+    def cache_spec(self):
+        specs = []
+        for _, m, _ in self.parts:
+            s = m.cache_spec()
+            specs += s if isinstance(s, list) else [s] if s else []
+        return specs
+
+    def mix(self, proj, b, cache, layer, out, out_scale=1.0):
+        i0 = o0 = 0
+        for _, m, scale in self.parts:
+            n = m.w_in.shape[0]
+            m.mix(proj[:, i0:i0 + n], b, cache, layer, out[:, o0:o0 + m.n_mid], out_scale * scale)
+            i0, o0 = i0 + n, o0 + m.n_mid
+        return out
+
+
+MIXERS = {c.kind: c for c in (GeneralDelta, Mamba2, LatentAttention, WindowAttention, GatedDelta,
+                              HGRN2, Parallel)}
 
 
 class DenseFF:
-    """Clamped gated feed-forward (``ops.seqmix.ff_act``)."""
+    """Gated feed-forward W_down(act(W_gate h) * W_up h): silu-gated, or with a ``limit`` in its
+    config the clamped unit of ``ops.seqmix.ff_act``."""
 
     def __init__(self, spec: dict, width: int):
         self.spec, self.width = spec, width
-        self.F, self.limit = int(spec["ff"]), float(spec["limit"])
+        self.F = int(spec["ff"])
+        self.limit = float(spec["limit"]) if spec.get("limit") is not None else None
 
     def tensor_shapes(self):
         return {"gate": (self.F, self.width), "up": (self.F, self.width), "down": (self.width, self.F)}
 
     def load(self, get, dtype, dev):
         self.w_gu = torch.cat([get("gate"), get("up")], 0).to(dev, dtype).contiguous()
+        self.w_in = self.w_gu
         self.w_down = get("down").to(dev, dtype).contiguous()
 
-    def forward(self, h):
-        gu = F.linear(h, self.w_gu)
-        act = torch.empty(h.shape[0], self.F, device=h.device, dtype=h.dtype)
-        sm.ff_act(gu, act, self.limit)
+    def forward_proj(self, gu):
+        """gu = [gate | up] projections of the input."""
+        act = torch.empty(gu.shape[0], self.F, device=gu.device, dtype=gu.dtype)
+        if self.limit is None:
+            sm.glu_act(gu, act)
+        else:
+            sm.ff_act(gu, act, self.limit)
         return F.linear(act, self.w_down)
+
+    def forward(self, h):
+        return self.forward_proj(F.linear(h, self.w_gu))
+
+
+class MoEFF:
+    """Mixture of clamped gated experts behind a sigmoid router whose choice is limited to
+    the best groups of experts (``ops.seqmix.group_route``); the chosen experts' scores weight
+    their outputs as they are.  The expert products run grouped over the routed rows
+    (``ops.seqmix.expert_gemm``)."""
+    w_in = None   # the router and the grouped products read the input themselves
+
+    def __init__(self, spec: dict, width: int):
+        self.spec, self.width = spec, width
+        r, e = spec["router"], spec["expert"]
+        self.E, self.top = int(r["experts"]), int(r["top"])
+        g = r.get("groups") or {}
+        self.groups, self.keep = int(g.get("count", 1)), int(g.get("keep", g.get("count", 1)))
+        self.F, self.limit = int(e["ff"]), float(e["limit"])
+        per = self.E // max(1, self.groups)
+        if self.groups < 1 or self.E % self.groups or not 1 <= self.keep <= self.groups \
+                or not 1 <= self.top <= self.keep * per:
+            raise ValueError("moe: %d experts in %d groups, %d kept, %d chosen"
+                             % (self.E, self.groups, self.keep, self.top))
+
+    def tensor_shapes(self):
+        d = {"router": (self.E, self.width)}
+        for e in range(self.E):
+            d.update({"e%d.gate" % e: (self.F, self.width), "e%d.up" % e: (self.F, self.width),
+                      "e%d.down" % e: (self.width, self.F)})
+        return d
+
+    def load(self, get, dtype, dev):
+        self.wr = get("router").to(dev).float().contiguous()
+        self.w_gu = torch.stack([torch.cat([get("e%d.gate" % e), get("e%d.up" % e)], 0)
+                                 for e in range(self.E)]).to(dev, dtype).contiguous()
+        self.w_down = torch.stack([get("e%d.down" % e) for e in range(self.E)]).to(dev, dtype).contiguous()
+
+    def forward(self, h):
+        R, top, dev = h.shape[0], self.top, h.device
+        ids = torch.empty(R, top, device=dev, dtype=torch.int32)
+        wts = torch.empty(R, top, device=dev, dtype=torch.float32)
+        cnt = torch.empty(self.E, device=dev, dtype=torch.int32)
+        rows = torch.empty(self.E, R * top, device=dev, dtype=torch.int32)
+        sm.group_route(h, self.wr, top, self.groups, self.keep, ids, wts, cnt, rows)
+        gu = torch.empty(R * top, 2 * self.F, device=dev, dtype=h.dtype)
+        sm.expert_gemm(h, top, self.w_gu, cnt, rows, gu, R * top)
+        act = torch.empty(R * top, self.F, device=dev, dtype=h.dtype)
+        sm.ff_act(gu, act, self.limit)
+        y = torch.empty(R * top, self.width, device=dev, dtype=h.dtype)
+        sm.expert_gemm(act, 1, self.w_down, cnt, rows, y, R * top)
+        out = torch.empty(R, self.width, device=dev, dtype=h.dtype)
+        return sm.expert_combine(y, wts, out)
+
+
+FEEDFORWARDS = {"dense": DenseFF, "moe": MoEFF}
 
 
 # ---------------------------------------------------------------------------- weights
 class HybridLayer:
     def __init__(self, spec: LayerSpec, cfg: HybridConfig):
+        self.block = cfg.traits.block
         self.mixer = MIXERS[spec.kind](spec.mixer, cfg.width, cfg.eps)
-        self.ff = DenseFF(spec.mlp, cfg.width) if spec.mlp is not None else None
+        self.ff = FEEDFORWARDS[spec.mlp.get("kind", "dense")](spec.mlp, cfg.width) \
+            if spec.mlp is not None else None
         self.norm1 = self.norm1b = self.ls1 = self.norm2 = self.norm2b = self.ls2 = None
+        # gated_post: the gates' projections ride on the sublayers' input products
+        self.w_in1 = self.w_in2 = self.rg1b = self.rg2b = None
 
     def tensor_shapes(self, W):
-        d = {"norm1": (W,), "norm1b": (W,), "ls1": (W,)}
+        gated = self.block == "gated_post"
+        d = {"norm1": (W,), "rg1": (W, W), "rg1.b": (W,)} if gated else \
+            {"norm1": (W,), "norm1b": (W,), "ls1": (W,)}
         d.update({"mix." + k: s for k, s in self.mixer.tensor_shapes().items()})
         if self.ff is not None:
-            d.update({"norm2": (W,), "norm2b": (W,), "ls2": (W,)})
+            d.update({"norm2": (W,), "rg2": (W, W), "rg2.b": (W,)} if gated else
+                     {"norm2": (W,), "norm2b": (W,), "ls2": (W,)})
             d.update({"mlp." + k: s for k, s in self.ff.tensor_shapes().items()})
         return d
+
+    def load(self, sd, p, dtype, dev):
+        self.mixer.load(lambda k: sd[p + "mix." + k], dtype, dev)
+        if self.ff is not None:
+            self.ff.load(lambda k: sd[p + "mlp." + k], dtype, dev)
+        if self.block == "gated_post":
+            if self.mixer.w_in is None:
+                raise ValueError("mixer %r cannot share its input product with a gate" % self.mixer.kind)
+            self.norm1, self.rg1b = _vec(sd[p + "norm1"], dev), _vec(sd[p + "rg1.b"], dev)
+            self.w_in1 = torch.cat([self.mixer.w_in, sd[p + "rg1"].to(dev, dtype)], 0).contiguous()
+            if self.ff is not None:
+                self.norm2, self.rg2b = _vec(sd[p + "norm2"], dev), _vec(sd[p + "rg2.b"], dev)
+                rg2 = sd[p + "rg2"].to(dev, dtype)
+                self.w_in2 = rg2.contiguous() if self.ff.w_in is None else \
+                    torch.cat([self.ff.w_in, rg2], 0).contiguous()
+            return
+        self.norm1, self.norm1b, self.ls1 = (_vec(sd[p + k], dev) for k in ("norm1", "norm1b", "ls1"))
+        if self.ff is not None:
+            self.norm2, self.norm2b, self.ls2 = (_vec(sd[p + k], dev) for k in ("norm2", "norm2b", "ls2"))
 
 
 def tensor_shapes(cfg: HybridConfig) -> dict:
     """name -> shape of every tensor of a checkpoint of this config."""
     W = cfg.width
-    d = {"embed": (cfg.vocab, W), "pos": (cfg.max_pos, W), "final.norm": (W,), "head": (cfg.vocab, W)}
+    d = {"embed": (cfg.vocab, W), "final.norm": (W,), "head": (cfg.vocab, W)}
+    if cfg.traits.positions:
+        d["pos"] = (cfg.max_pos, W)
     for i, spec in enumerate(cfg.layers):
         d.update({"l%d.%s" % (i, k): s for k, s in HybridLayer(spec, cfg).tensor_shapes(W).items()})
     return d
@@ -392,18 +735,13 @@ class HybridWeights:
             if tuple(sd[k].shape) != tuple(s):
                 raise ValueError("tensor %r has shape %s, the config gives %s" % (k, tuple(sd[k].shape), s))
         self.embed = sd["embed"].to(dev, dtype).contiguous()
-        self.pos = sd["pos"].to(dev, dtype).contiguous()
+        self.pos = sd["pos"].to(dev, dtype).contiguous() if cfg.traits.positions else None
         self.final_norm = _vec(sd["final.norm"], dev)
         self.head = sd["head"].to(dev, dtype).contiguous()
         self.layers = []
         for i, spec in enumerate(cfg.layers):
             L = HybridLayer(spec, cfg)
-            p = "l%d." % i
-            L.mixer.load(lambda k, p=p: sd[p + "mix." + k], dtype, dev)
-            L.norm1, L.norm1b, L.ls1 = (_vec(sd[p + k], dev) for k in ("norm1", "norm1b", "ls1"))
-            if L.ff is not None:
-                L.ff.load(lambda k, p=p: sd[p + "mlp." + k], dtype, dev)
-                L.norm2, L.norm2b, L.ls2 = (_vec(sd[p + k], dev) for k in ("norm2", "norm2b", "ls2"))
+            L.load(sd, "l%d." % i, dtype, dev)
             self.layers.append(L)
 
     @classmethod
@@ -421,12 +759,14 @@ def random_state_dict(cfg: HybridConfig, seed: int = 0) -> dict:
     sd = {}
     for k, s in tensor_shapes(cfg).items():
         leaf = k.split(".", 1)[1] if k.startswith("l") and "." in k else k
-        if len(s) == 2 and not leaf.endswith("mix.conv"):
+        if len(s) == 2 and not leaf.endswith("conv"):
             t = torch.randn(*s, generator=g) / (s[1] ** 0.5 if k not in ("embed", "pos") else 1.0)
-        elif leaf.endswith("mix.conv"):
+        elif leaf.endswith("conv"):
             t = torch.randn(*s, generator=g) * 0.5
-        elif leaf.endswith(("norm1", "norm2", "norm1b", "norm2b", "mix.norm", "dkv.norm")) or k == "final.norm":
+        elif leaf.endswith(("norm1", "norm2", "norm1b", "norm2b", ".norm")) or k == "final.norm":
             t = 1.0 + 0.1 * torch.randn(*s, generator=g)
+        elif leaf.endswith("lower"):
+            t = torch.rand(*s, generator=g) * 0.9
         elif leaf in ("ls1", "ls2"):
             t = 0.5 + 0.1 * torch.randn(*s, generator=g)
         elif leaf.endswith("A_log"):
@@ -464,6 +804,8 @@ class HybridModel:
         cfg, w = self.cfg, self.w
         if b.max_pos >= cfg.max_pos:
             raise ValueError("position %d exceeds the model's %d positions" % (b.max_pos, cfg.max_pos))
+        if cfg.traits.block == "gated_post":
+            return self._forward_gated_post(b, layer_out)
         x = torch.empty(b.R, cfg.width, device=self.device, dtype=torch.float32)
         sm.embed_pos(w.embed, w.pos, b.ids, b.pos, x)
         h = torch.empty(b.R, cfg.width, device=self.device, dtype=self.dtype)
@@ -482,6 +824,44 @@ class HybridModel:
                 layer_out.append(x.clone())
         if b.n_out == 0:
             return None
+        return self._logits(x, b)
+
+    def _logits(self, x, b: StepBatch):
+        cfg, w = self.cfg, self.w
         hn = torch.empty(b.n_out, cfg.width, device=self.device, dtype=self.dtype)
-        sm.rmsnorm(x, w.final_norm, cfg.eps, hn, in_rows=b.out_rows)
-        return F.linear(hn, w.head).float()
+        sm.rmsnorm(x, w.final_norm, cfg.eps, hn, parts=cfg.norm_groups, in_rows=b.out_rows)
+        y = F.linear(hn, w.head)
+        if not cfg.logit_softcap:
+            return y.float()
+        return sm.softcap(y, cfg.logit_softcap, torch.empty(y.shape, device=y.device, dtype=torch.float32))
+
+    def _forward_gated_post(self, b: StepBatch, layer_out=None):
+        """x <- x + N(f(x) * sigmoid(R x + b)) per sublayer: the sublayer and its gate read the
+        residual rows as they are (rounded to the activation type), so one matrix product
+        serves both; the pass that adds the result also writes the next sublayer's input."""
+        cfg, w = self.cfg, self.w
+        x = torch.empty(b.R, cfg.width, device=self.device, dtype=torch.float32)
+        # in float32 the sublayers read the residual stream itself
+        h = x if self.dtype == torch.float32 else \
+            torch.empty(b.R, cfg.width, device=self.device, dtype=self.dtype)
+        nxt = None if h is x else h
+        sm.embed_rows(w.embed, b.ids, x, nxt)
+        parts, eps = cfg.norm_groups, cfg.eps
+        for i, L in enumerate(w.layers):
+            n = L.mixer.w_in.shape[0]
+            proj = F.linear(h, L.w_in1)
+            m = L.mixer.forward_proj(proj[:, :n], b, self.cache, i)
+            sm.gate_norm_add(x, m, proj[:, n:], L.rg1b, L.norm1, parts, eps, next_out=nxt)
+            if L.ff is not None:
+                proj = F.linear(h, L.w_in2)
+                if L.ff.w_in is None:
+                    f, gate = L.ff.forward(h), proj
+                else:
+                    n = L.ff.w_in.shape[0]
+                    f, gate = L.ff.forward_proj(proj[:, :n]), proj[:, n:]
+                sm.gate_norm_add(x, f, gate, L.rg2b, L.norm2, parts, eps, next_out=nxt)
+            if layer_out is not None:
+                layer_out.append(x.clone())
+        if b.n_out == 0:
+            return None
+        return self._logits(x, b)

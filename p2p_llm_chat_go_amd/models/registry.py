@@ -1,7 +1,7 @@
 """Model registry: which config, weight store and engine serve a checkpoint or preset.
 
 A checkpoint folder is recognised by its ``config.json``: an ``architecture`` key naming a
-hybrid design (``HYBRID_ARCHITECTURES``) selects ``models.hybrid`` + ``engine.hybrid``;
+hybrid design (``models.hybrid.DESIGNS``) selects ``models.hybrid`` + ``engine.hybrid``;
 anything else is read as an HF Llama / Mixtral config (``models.weights``) for ``Engine``.
 """
 from __future__ import annotations
@@ -11,12 +11,15 @@ import os
 
 import torch
 
-HYBRID_ARCHITECTURES = ("Regesun",)
+def hybrid_architectures() -> tuple:
+    from .hybrid import DESIGNS
+
+    return tuple(DESIGNS)
 
 
 def is_hybrid_dir(path: str) -> bool:
     with open(os.path.join(path, "config.json")) as f:
-        return json.load(f).get("architecture") in HYBRID_ARCHITECTURES
+        return json.load(f).get("architecture") in hybrid_architectures()
 
 
 def supports_dtype(path: str, dtype) -> bool:

@@ -63,6 +63,34 @@ _SIGS = {
                             c_int, c_int, c_int, c_void_p],
     "p2p_sm_ff_act": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_float, c_int,
                       c_void_p],
+    "p2p_sm_gate_norm_add": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
+                             c_int, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
+    "p2p_sm_glu_act": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "p2p_sm_softcap": [c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_int, c_void_p],
+    "p2p_sm_embed_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                          c_void_p],
+    "p2p_sm_qk_norm_rope_store": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
+                                  c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_float,
+                                  c_void_p, c_int, c_int, c_int, c_void_p],
+    "p2p_sm_window_attn": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                           c_void_p, c_float, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                           c_int, c_int, c_float, c_int, c_void_p],
+    "p2p_sm_window_attn_mfma": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                c_void_p, c_int, c_void_p, c_float, c_int, c_void_p, c_int, c_int,
+                                c_int, c_int, c_int, c_int, c_int, c_void_p, c_float, c_void_p],
+    "p2p_sm_hgrn2_scan": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                          c_int, c_void_p, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
+                          c_void_p],
+    "p2p_sm_gated_delta_scan": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p,
+                                c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float,
+                                c_int, c_void_p],
+    "p2p_sm_group_route": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                           c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "p2p_sm_expert_gemm": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                           c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "p2p_sm_expert_combine": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                              c_int, c_void_p],
 }
 
 _lock = threading.Lock()
@@ -159,6 +187,27 @@ def embed_pos(embed, pos_table, ids, pos, out):
     _chk(lib().p2p_sm_embed_pos(embed.data_ptr(), _lib.ptr(pos_table), ids.data_ptr(),
                                 pos.data_ptr(), out.data_ptr(), R, W, _f32(embed), _st(out)),
          "embed_pos")
+    return out
+
+
+def embed_rows(embed, ids, out, h_out=None):
+    """out[r] = embed[ids[r]] as fp32 rows; h_out (activation type, optional): the same rows
+    for a first sublayer that reads the residual stream as it is."""
+    R, W = out.shape
+    if not out.is_cuda:
+        out.copy_(embed[ids[:R].long()].float())
+        if h_out is not None:
+            h_out[:R] = out.to(h_out.dtype)
+        return out
+    assert out.dtype == torch.float32 and out.is_contiguous() and embed.shape[1] == W
+    assert ids.dtype == torch.int32 and ids.numel() >= R and embed.is_contiguous()
+    ldh = 0
+    if h_out is not None:
+        _rows2d(h_out, "h_out")
+        assert h_out.dtype == embed.dtype and h_out.shape[1] == W and h_out.shape[0] >= R
+        ldh = h_out.stride(0)
+    _chk(lib().p2p_sm_embed_rows(embed.data_ptr(), ids.data_ptr(), out.data_ptr(),
+                                 _lib.ptr(h_out), ldh, R, W, _f32(embed), _st(out)), "embed_rows")
     return out
 
 
@@ -378,6 +427,28 @@ def mamba_conv(zx, xoff: int, cw, cb, tail, ent, ent_host, row_ent, out):
     return out
 
 
+def conv_tail_roll(zx, xoff: int, tail, ent, ent_host, C: int):
+    """After a step's convolutions: every entry's slot keeps the raw inputs (channels
+    [xoff, xoff + C) of zx) of its last K-1 tokens, older ones shifted out.  tail fp32
+    [slots, K-1, C]."""
+    Km1 = tail.shape[1]
+    if Km1 == 0:
+        return tail
+    if not zx.is_cuda:
+        for row0, n, start, slot in ent_host:
+            raw = zx[row0:row0 + n, xoff:xoff + C].float()
+            prev = tail[slot] if start > 0 else torch.zeros(Km1, C)
+            tail[slot] = torch.cat([prev, raw], 0)[-Km1:]
+        return tail
+    _rows2d(zx, "zx")
+    assert tail.dtype == torch.float32 and tail.is_contiguous() and tail.shape[2] == C
+    assert xoff + C <= zx.shape[1]
+    _chk(lib().p2p_sm_mamba_tail(zx.data_ptr(), zx.stride(0), xoff, tail.data_ptr(),
+                                 ent.data_ptr(), ent.shape[0], C, Km1 + 1, _f32(zx), _st(zx)),
+         "conv_tail_roll")
+    return tail
+
+
 def mamba_scan(conv, zx, xoff: int, dtoff: int, dt_bias, A_log, Dp, state, tail, ent, ent_host,
                y, H: int, P: int, N: int, G: int):
     """Selective state-space scan.  conv fp32 [R, H*P + 2*G*N] = silu(conv(x | B | C)); zx the
@@ -538,4 +609,376 @@ def latent_attn(qa, cache, block_tables, row_ent, pos, sink, scale: float, win: 
                                   row_ent.data_ptr(), pos.data_ptr(), sink.data_ptr(), scale,
                                   win, out.data_ptr(), out.stride(0), out.stride(1), R, H, rank,
                                   page, _f32(qa), _st(qa)), "latent_attn")
+    return out
+
+
+# ------------------------------------------------------------------ post-norm gated residual
+def gate_norm_add(x, y, g, gb, w, parts: int, eps: float, next_out=None):
+    """x += N(y * sigmoid(g + gb)) * w on the fp32 residual x, N the RMS norm taken separately
+    over ``parts`` equal parts of the row.  y, g: activation-typed [R, n] (g the gate's
+    projection before its bias gb).  next_out (activation type): the updated rows, which the
+    next sublayer reads as they are."""
+    R, n = x.shape
+    if not x.is_cuda:
+        v = y.float() * torch.sigmoid(g.float() + gb)
+        x += _rms(v.view(R, parts, n // parts), eps).reshape(R, n) * w
+        if next_out is not None:
+            next_out[:R] = x.to(next_out.dtype)
+        return x
+    _rows2d(y, "y")
+    _rows2d(g, "g")
+    assert x.dtype == torch.float32 and x.is_contiguous() and y.shape == x.shape == g.shape
+    assert y.dtype == g.dtype
+    _vec(w, n, "w")
+    _vec(gb, n, "gb")
+    if parts < 1 or n % parts:
+        raise ValueError("row of %d does not split into %d parts" % (n, parts))
+    ldh = 0
+    if next_out is not None:
+        _rows2d(next_out, "next_out")
+        assert next_out.shape[1] == n and next_out.shape[0] >= R
+        ldh = next_out.stride(0)
+    _chk(lib().p2p_sm_gate_norm_add(x.data_ptr(), y.data_ptr(), y.stride(0), g.data_ptr(),
+                                    g.stride(0), gb.data_ptr(), w.data_ptr(), R, n, parts, eps,
+                                    _lib.ptr(next_out), ldh,
+                                    _f32(next_out) if next_out is not None else 0, _f32(y),
+                                    _st(x)), "gate_norm_add")
+    return x
+
+
+def glu_act(gu, out):
+    """[gate | up] -> silu(gate) * up."""
+    R, F = out.shape
+    if not gu.is_cuda:
+        g = gu[:, :F].float()
+        out.copy_((g * torch.sigmoid(g) * gu[:, F:].float()).to(out.dtype))
+        return out
+    _rows2d(gu, "gu")
+    _rows2d(out, "out")
+    assert gu.shape == (R, 2 * F) and gu.dtype == out.dtype
+    _chk(lib().p2p_sm_glu_act(gu.data_ptr(), gu.stride(0), out.data_ptr(), out.stride(0), R, F,
+                              _f32(gu), _st(gu)), "glu_act")
+    return out
+
+
+def softcap(y, cap: float, out):
+    """out = cap * tanh(y / cap) as fp32 (y: activation-typed or fp32 logits)."""
+    if not y.is_cuda:
+        out.copy_(cap * torch.tanh(y.float() / cap))
+        return out
+    _rows2d(y, "y")
+    assert out.dtype == torch.float32 and out.is_contiguous() and out.shape == y.shape
+    _chk(lib().p2p_sm_softcap(y.data_ptr(), y.stride(0), out.data_ptr(), y.shape[0], y.shape[1],
+                              cap, _f32(y), _st(y)), "softcap")
+    return out
+
+
+# ------------------------------------------------------------------ windowed attention
+def rope_inv_freq(base: float, dims: int, device) -> torch.Tensor:
+    """f_i = base^(-2i/dims), i < dims/2, evaluated in float64 and rounded to fp32."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).float().to(device)
+
+
+def qk_norm_rope_store(proj, H: int, G: int, D: int, V: int, qw, kw, inv_freq, pos, cache_rows,
+                       pool, eps: float, q_out):
+    """Prepares attention inputs from one projection buffer proj = [q (H*D) | k (G*D) | v (G*V)]:
+    q and k are RMS-normalised over their whole rows (all heads at once) with weights qw / kw,
+    then channels (2i, 2i+1), i < len(inv_freq), of every head are rotated by pos * inv_freq[i].
+    q goes to q_out [R, H*D]; k | v go to the paged pool rows ``cache_rows`` ([tokens,
+    G*D + G*V]).  Norm, angles and the rotation are fp32."""
+    R = q_out.shape[0]
+    nq, nk, nv = H * D, G * D, G * V
+    nrot = inv_freq.numel()
+    if not proj.is_cuda:
+        ang = (pos[:R].float()[:, None] * inv_freq[None, :])
+        c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+
+        def rot(t, heads):
+            t = t.view(R, heads, D).clone()
+            u, v = t[:, :, 0:2 * nrot:2].clone(), t[:, :, 1:2 * nrot:2].clone()
+            t[:, :, 0:2 * nrot:2] = u * c - v * s
+            t[:, :, 1:2 * nrot:2] = v * c + u * s
+            return t.reshape(R, heads * D)
+
+        q = rot(_rms(proj[:R, :nq].float(), eps) * qw, H)
+        k = rot(_rms(proj[:R, nq:nq + nk].float(), eps) * kw, G)
+        q_out[:R] = q.to(q_out.dtype)
+        rows = cache_rows[:R].long()
+        pool[rows, :nk] = k.to(pool.dtype)
+        pool[rows, nk:] = proj[:R, nq + nk:nq + nk + nv].to(pool.dtype)
+        return q_out
+    _rows2d(proj, "proj")
+    _rows2d(q_out, "q_out")
+    assert proj.shape[1] >= nq + nk + nv and q_out.shape[1] == nq and q_out.dtype == proj.dtype
+    assert pool.dim() == 2 and pool.is_contiguous() and pool.shape[1] == nk + nv
+    assert pool.dtype == proj.dtype
+    _vec(qw, nq, "qw")
+    _vec(kw, nk, "kw")
+    assert inv_freq.dtype == torch.float32 and inv_freq.is_contiguous() and 2 * nrot <= D
+    assert pos.dtype == torch.int32 and cache_rows.dtype == torch.int32
+    _chk(lib().p2p_sm_qk_norm_rope_store(proj.data_ptr(), proj.stride(0), H, G, D, V,
+                                         qw.data_ptr(), kw.data_ptr(), inv_freq.data_ptr(), nrot,
+                                         pos.data_ptr(), cache_rows.data_ptr(), pool.data_ptr(),
+                                         eps, q_out.data_ptr(), q_out.stride(0), R, _f32(proj),
+                                         _st(proj)), "qk_norm_rope_store")
+    return q_out
+
+
+def window_rows_per_wave(HG: int) -> int:
+    """Rows of one sequence portion that a wavefront of the matrix-core window attention takes:
+    its 16 (row, head) pairs are RW rows x HS slots for the HG query heads of a key/value head."""
+    return latent_rows_per_wave(HG)
+
+
+def window_mfma_ok(q, pool, D: int, V: int) -> bool:
+    """The matrix-core kernel serves bf16 with key / value sizes that are multiples of 8 up to
+    256 and 16-byte aligned rows.  P2P_WINDOW_MFMA=0 switches it off."""
+    return (q.is_cuda and q.dtype == torch.bfloat16 and D % 8 == 0 and V % 8 == 0
+            and 8 <= D <= 256 and 8 <= V <= 256 and q.stride(0) % 8 == 0
+            and q.data_ptr() % 16 == 0 and pool.data_ptr() % 16 == 0 and pool.shape[1] % 8 == 0
+            and os.environ.get("P2P_WINDOW_MFMA", "1") != "0")
+
+
+def window_attn(q, pool, block_tables, row_ent, pos, sink, scale: float, win: int, out, page: int,
+                H: int, G: int, D: int, V: int, units=None, max_keys=None, out_scale: float = 1.0):
+    """Grouped-query attention over a paged key/value pool with a causal sliding window and a
+    softmax sink.
+
+    q [R, H*D] (rotated), pool [tokens, G*D + G*V] (token t of a sequence at
+    block_tables[e, t // page] * page + t % page; keys first, then values), query head h reads
+    key/value head h // (H/G).  out [R, H*V] = sum_j p_j v_j with
+    p = softmax over {sink_h} U {scale * q . k_j : 0 <= pos - j < win}; the sink has no value;
+    the result is multiplied by out_scale before it is rounded.
+    units: ``make_units(entries, window_rows_per_wave(H // G))`` on the device; with it bf16
+    inputs run on the matrix cores (``window_mfma_ok``)."""
+    R = q.shape[0]
+    HG = H // G
+    if not q.is_cuda:
+        bt = block_tables.long()
+        for r in range(R):
+            p = int(pos[r])
+            lo = max(0, p - win + 1)
+            j = torch.arange(lo, p + 1)
+            tok = bt[int(row_ent[r])][j // page] * page + j % page
+            kv = pool[tok].float()
+            k = kv[:, :G * D].view(-1, G, D).repeat_interleave(HG, 1)       # [n, H, D]
+            v = kv[:, G * D:].view(-1, G, V).repeat_interleave(HG, 1)
+            s = torch.einsum("hd,nhd->hn", q[r].float().view(H, D), k) * scale
+            m = torch.maximum(s.max(-1).values, sink)
+            e = torch.exp(s - m[:, None])
+            den = e.sum(-1) + torch.exp(sink - m)
+            out[r] = (torch.einsum("hn,nhv->hv", e / den[:, None], v).reshape(H * V) * out_scale).to(out.dtype)
+        return out
+    _rows2d(q, "q")
+    _rows2d(out, "out")
+    assert H % G == 0 and q.shape[1] == H * D and out.shape == (R, H * V)
+    assert q.dtype == pool.dtype == out.dtype
+    assert pool.dim() == 2 and pool.is_contiguous() and pool.shape[1] == G * (D + V)
+    assert block_tables.dtype == torch.int32 and block_tables.is_contiguous()
+    assert row_ent.dtype == torch.int32 and pos.dtype == torch.int32
+    _vec(sink, H, "sink")
+    if win < 1:
+        raise ValueError("window of %d keys" % win)
+    if units is not None and window_mfma_ok(q, pool, D, V):
+        assert units.dtype == torch.int32 and units.is_contiguous() and units.shape[1] == 2
+        U = units.shape[0]
+        hs = 16 // window_rows_per_wave(HG)
+        blocks = U * G * (-(-HG // hs))
+        splits = 1
+        if max_keys is not None and blocks < LATENT_SPLIT_BLOCKS:
+            splits = max(1, min(-(-min(max_keys, win) // 64), LATENT_SPLIT_BLOCKS // blocks, 64))
+        part = None
+        if splits > 1:
+            L = lib()
+            L.p2p_sm_window_attn_mfma_ws.restype = c_long
+            part = torch.empty(L.p2p_sm_window_attn_mfma_ws(U, H, G, V, splits), device=q.device,
+                               dtype=torch.float32)
+        _chk(lib().p2p_sm_window_attn_mfma(q.data_ptr(), q.stride(0), pool.data_ptr(),
+                                           block_tables.data_ptr(), block_tables.shape[1],
+                                           row_ent.data_ptr(), pos.data_ptr(), units.data_ptr(), U,
+                                           sink.data_ptr(), scale, win, out.data_ptr(),
+                                           out.stride(0), H, G, D, V, page, splits, _lib.ptr(part),
+                                           out_scale, _st(q)), "window_attn_mfma")
+        return out
+    _chk(lib().p2p_sm_window_attn(q.data_ptr(), q.stride(0), pool.data_ptr(),
+                                  block_tables.data_ptr(), block_tables.shape[1],
+                                  row_ent.data_ptr(), pos.data_ptr(), sink.data_ptr(), scale, win,
+                                  out.data_ptr(), out.stride(0), R, H, G, D, V, page, out_scale,
+                                  _f32(q), _st(q)), "window_attn")
+    return out
+
+
+# ------------------------------------------------------------------ gated linear scans
+# Per head a D x V fp32 state S (key channel i, value channel j), one step per token:
+#   S <- diag(g) S;   u = v                      (plain write)
+#                     u = beta * (v - S^T k)     (delta rule: the write corrects what k reads)
+#   S <- S + k u^T;   o = S^T q                  (the read-out sees the token's own write)
+# HGRN2 is the plain write with g = f and k = 1 - f; the gated delta rule has its own key.
+def hgrn2_scan(proj, lower, fb, normw, state, ent, ent_host, out, H: int, D: int, V: int,
+               eps: float, out_scale: float = 1.0):
+    """proj = [q (H*D) | f (H*D) | v (H*V)] raw projections of the step's rows.  q = silu(q),
+    f = lower + (1 - lower) * sigmoid(f + fb); S <- diag(f) S + (1 - f) v^T; o = S^T q; every
+    head's o is RMS-normalised over V and weighted by normw [V].  state fp32 [slots, H, D, V];
+    out [R, H*V] activation type."""
+    n = H * D
+    if not proj.is_cuda:
+        for row0, cnt, start, slot in ent_host:
+            S = state[slot] if start > 0 else torch.zeros_like(state[slot])
+            for t in range(row0, row0 + cnt):
+                qr = proj[t, :n].float()
+                q = (qr * torch.sigmoid(qr)).view(H, D)
+                f = (lower + (1 - lower) * torch.sigmoid(proj[t, n:2 * n].float() + fb)).view(H, D)
+                v = proj[t, 2 * n:2 * n + H * V].float().view(H, V)
+                S = f[:, :, None] * S + (1 - f)[:, :, None] * v[:, None, :]
+                o = torch.einsum("hdv,hd->hv", S, q)
+                out[t] = (_rms(o, eps) * normw * out_scale).reshape(H * V).to(out.dtype)
+            state[slot] = S
+        return out
+    _rows2d(proj, "proj")
+    _rows2d(out, "out")
+    assert proj.shape[1] >= 2 * n + H * V and out.shape[1] == H * V and out.dtype == proj.dtype
+    _vec(lower, n, "lower")
+    _vec(fb, n, "fb")
+    _vec(normw, V, "normw")
+    _scan_state_ok(state, H, D, V, ent)
+    _chk(lib().p2p_sm_hgrn2_scan(proj.data_ptr(), proj.stride(0), lower.data_ptr(), fb.data_ptr(),
+                                 normw.data_ptr(), state.data_ptr(), ent.data_ptr(), ent.shape[0],
+                                 out.data_ptr(), out.stride(0), H, D, V, eps, out_scale,
+                                 _f32(proj), _st(proj)), "hgrn2_scan")
+    return out
+
+
+def _scan_state_ok(state, H, D, V, ent):
+    assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, D, V)
+    assert ent.dtype == torch.int32 and ent.is_contiguous() and ent.shape[1] == 4
+    if D > 256 or V > 256:
+        raise ValueError("gated scan: key %d / value %d sizes above 256" % (D, V))
+
+
+def gated_delta_scan(conv, araw, braw, gate, A_log, dt_bias, normw, state, ent, ent_host, out,
+                     H: int, G: int, D: int, V: int, eps: float, out_scale: float = 1.0):
+    """Gated delta rule.  conv fp32 [R, 2*G*D + H*V] = silu(conv(q | k | v)); q and k become
+    unit vectors per head (x / sqrt(|x|^2 + 1e-6)), q also times D^-1/2; head h reads q/k head
+    h // (H/G).  araw [R, H*D]: decay logits, g = exp(-exp(A_log_h) * softplus(araw + dt_bias));
+    braw [R, H]: beta = sigmoid(braw); gate [R, H*V]: the output gate's logits.  Every head's
+    o is RMS-normalised over V, weighted by normw [V] and multiplied by sigmoid(gate).
+    state fp32 [slots, H, D, V]; out [R, H*V] activation type."""
+    R = out.shape[0]
+    hg = H // G
+    if not conv.is_cuda:
+        nA = torch.exp(A_log)
+        for row0, cnt, start, slot in ent_host:
+            S = state[slot] if start > 0 else torch.zeros_like(state[slot])
+            for t in range(row0, row0 + cnt):
+                q = conv[t, :G * D].view(G, D)
+                k = conv[t, G * D:2 * G * D].view(G, D)
+                v = conv[t, 2 * G * D:].view(H, V)
+                q = (q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * D ** -0.5).repeat_interleave(hg, 0)
+                k = (k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)).repeat_interleave(hg, 0)
+                dt = torch.nn.functional.softplus(araw[t].float() + dt_bias, threshold=1e9).view(H, D)
+                g = torch.exp(-nA[:, None] * dt)
+                beta = torch.sigmoid(braw[t].float())
+                S = g[:, :, None] * S
+                u = beta[:, None] * (v - torch.einsum("hdv,hd->hv", S, k))
+                S = S + k[:, :, None] * u[:, None, :]
+                o = torch.einsum("hdv,hd->hv", S, q)
+                o = _rms(o, eps) * normw * torch.sigmoid(gate[t].float()).view(H, V)
+                out[t] = (o.reshape(H * V) * out_scale).to(out.dtype)
+            state[slot] = S
+        return out
+    assert conv.dtype == torch.float32 and conv.is_contiguous() and conv.shape[1] == 2 * G * D + H * V
+    for t_, nm, n in ((araw, "araw", H * D), (braw, "braw", H), (gate, "gate", H * V), (out, "out", H * V)):
+        _rows2d(t_, nm)
+        assert t_.shape[1] == n and t_.dtype == out.dtype, nm
+    _vec(A_log, H, "A_log")
+    _vec(dt_bias, H * D, "dt_bias")
+    _vec(normw, V, "normw")
+    assert H % G == 0
+    _scan_state_ok(state, H, D, V, ent)
+    _chk(lib().p2p_sm_gated_delta_scan(conv.data_ptr(), conv.stride(0), araw.data_ptr(),
+                                       araw.stride(0), braw.data_ptr(), braw.stride(0),
+                                       gate.data_ptr(), gate.stride(0), A_log.data_ptr(),
+                                       dt_bias.data_ptr(), normw.data_ptr(), state.data_ptr(),
+                                       ent.data_ptr(), ent.shape[0], out.data_ptr(), out.stride(0),
+                                       H, G, D, V, eps, out_scale, _f32(out), _st(out)),
+         "gated_delta_scan")
+    return out
+
+
+# ------------------------------------------------------------------ mixture of experts
+def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows):
+    """Sigmoid router with group-limited choice.  z = h wr^T in fp32 (wr fp32 [E, W]),
+    s = sigmoid(z); the E experts form ``groups`` equal groups of neighbours, a group scores the
+    sum of its two largest s, only experts of the best ``keep`` groups can be chosen; the
+    ``top`` largest s among them win (ties: the lower index), their weights are their s.
+    ids int32 / wts fp32 [R, top]; cnt int32 [E] and rows int32 [E, R*top] list per expert the
+    slots (row * top + k) routed to it (cnt is cleared here)."""
+    R = h.shape[0]
+    E = wr.shape[0]
+    per = E // groups
+    if not h.is_cuda:
+        s = torch.sigmoid(h.float() @ wr.t())                                     # [R, E]
+        gs = s.view(R, groups, per).topk(min(2, per), dim=-1).values.sum(-1)      # [R, groups]
+        best = gs.topk(keep, dim=-1).indices
+        ok = torch.zeros(R, groups, dtype=torch.bool).scatter_(1, best, True)
+        masked = torch.where(ok.repeat_interleave(per, 1), s, torch.full_like(s, -1.0))
+        w, i = masked.topk(top, dim=-1)
+        ids[:R] = i.to(torch.int32)
+        wts[:R] = w
+        cnt.zero_()
+        for slot, e in enumerate(i.reshape(-1).tolist()):
+            rows[e, int(cnt[e])] = slot
+            cnt[e] += 1
+        return ids, wts
+    _rows2d(h, "h")
+    assert wr.dtype == torch.float32 and wr.is_contiguous() and wr.shape[1] == h.shape[1]
+    assert E % groups == 0 and 1 <= keep <= groups and 1 <= top <= keep * per
+    if E > 1024:
+        raise ValueError("group_route: %d experts > 1024" % E)
+    assert ids.dtype == torch.int32 and ids.is_contiguous() and ids.shape == (R, top)
+    assert wts.dtype == torch.float32 and wts.is_contiguous() and wts.shape == (R, top)
+    assert cnt.dtype == torch.int32 and cnt.numel() == E
+    assert rows.dtype == torch.int32 and rows.is_contiguous() and rows.shape[0] == E \
+        and rows.shape[1] >= R * top
+    cnt.zero_()
+    _chk(lib().p2p_sm_group_route(h.data_ptr(), h.stride(0), wr.data_ptr(), R, h.shape[1], E, top,
+                                  groups, keep, ids.data_ptr(), wts.data_ptr(), cnt.data_ptr(),
+                                  rows.data_ptr(), rows.stride(0), _f32(h), _st(h)), "group_route")
+    return ids, wts
+
+
+def expert_gemm(x, x_div: int, w, cnt, rows, out, max_slots: int):
+    """Per expert e and each of its routed slots s = rows[e, i] (i < cnt[e]):
+    out[s] = x[s // x_div] @ w[e]^T.  w [E, N, K] (activation type), x [*, K], out [slots, N].
+    Accumulation is fp32; a slot's result does not depend on the other slots."""
+    E, N, K = w.shape
+    if not x.is_cuda:
+        for e in range(E):
+            sl = rows[e, :int(cnt[e])].long()
+            if sl.numel():
+                out[sl] = torch.nn.functional.linear(x[sl // x_div], w[e])
+        return out
+    _rows2d(x, "x")
+    _rows2d(out, "out")
+    assert w.is_contiguous() and x.shape[1] == K and out.shape[1] == N
+    assert x.dtype == w.dtype == out.dtype and rows.stride(0) >= max_slots
+    _chk(lib().p2p_sm_expert_gemm(x.data_ptr(), x.stride(0), x_div, w.data_ptr(), cnt.data_ptr(),
+                                  rows.data_ptr(), rows.stride(0), out.data_ptr(), out.stride(0),
+                                  E, N, K, max_slots, _f32(x), _st(x)), "expert_gemm")
+    return out
+
+
+def expert_combine(y, wts, out):
+    """out[r] = sum_k wts[r, k] * y[r * top + k] (fp32 sum, activation-typed result)."""
+    R, top = wts.shape
+    if not y.is_cuda:
+        out[:R] = (y[:R * top].float().view(R, top, -1) * wts[:, :, None]).sum(1).to(out.dtype)
+        return out
+    _rows2d(y, "y")
+    _rows2d(out, "out")
+    assert y.shape[0] >= R * top and out.shape[1] == y.shape[1] and y.dtype == out.dtype
+    _chk(lib().p2p_sm_expert_combine(y.data_ptr(), y.stride(0), wts.data_ptr(), out.data_ptr(),
+                                     out.stride(0), R, top, y.shape[1], _f32(y), _st(y)),
+         "expert_combine")
     return out
