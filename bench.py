@@ -68,8 +68,13 @@ def parse(argv=None):
                     help="cpu: gloo + the CPU engine (plumbing tests with tiny models)")
     ap.add_argument("--hybrid", action="store_true",
                     help="instead of the headline workload: prefill / decode throughput of "
-                         "Regesun hybrid models beside a dense Llama of equal size "
+                         "hybrid models (Regesun, Rotutar) beside a dense Llama of equal size "
                          "(bench/hybrid_bench.py; 1 GPU)")
+    ap.add_argument("--hybrid-design", choices=("regesun", "rotutar", "both"), default="regesun",
+                    help="regesun: Regesun beside the Llama; rotutar: Rotutar beside Regesun "
+                         "(equal width and depth); both: all three")
+    ap.add_argument("--hybrid-only", default=None,
+                    help="run only the models whose name contains this (profiling one model)")
     ap.add_argument("--hybrid-sizes", default="1024,2048", help="model widths for --hybrid")
     ap.add_argument("--hybrid-prompt", type=int, default=2048)
     ap.add_argument("--hybrid-batch", type=int, default=8)

@@ -1,8 +1,12 @@
-"""Prefill and decode throughput of hybrid (Regesun) models at layer sizes that resemble real
-models, beside a dense Llama of the same width, depth and parameter count on the same engine
-entry point (``generate``).  Random weights, random tokens.
+"""Prefill and decode throughput of hybrid models (Regesun, Rotutar) at layer sizes that
+resemble real models, beside a dense Llama of the same width, depth and parameter count on
+the same engine entry point (``generate``).  Random weights, random tokens.
 
-    python bench.py --hybrid [--hybrid-sizes 1024,2048] [--steps K] [--warmup W]
+    python bench.py --hybrid [--hybrid-design regesun|rotutar|both] [--hybrid-sizes 1024,2048]
+                    [--steps K] [--warmup W]
+
+``--hybrid-design rotutar`` runs Rotutar beside Regesun (the closest model: same engine, same
+width and depth) instead of the Llama.
 
 One JSON line per (size, model): prefill tokens/s of one long prompt (``prompt`` tokens),
 decode tokens/s of ``batch`` sequences.  These lines are not the headline metric.
@@ -30,6 +34,30 @@ def regesun_config(width: int):
     return HybridConfig.from_dict(
         {"architecture": "Regesun", "width": width, "vocab": 32000, "max_positions": 8192,
          "norm": {"eps": 1e-5}, "layers": [gd, mb, mb, la] * 4}, name="regesun-w%d" % width)
+
+
+def rotutar_config(width: int):
+    """A Rotutar stack at a given width: blocks of hgrn2 / hgrn2+moe / hgrn2 / (window attention
+    beside the gated delta rule)+dense ff, 128-wide heads."""
+    from p2p_llm_chat_go_amd.models.hybrid import HybridConfig
+
+    hd = 128
+    nh = width // hd
+    moe = {"kind": "moe", "expert": {"ff": width // 2, "limit": 7.0},
+           "router": {"experts": 8, "top": 2, "groups": {"count": 4, "keep": 2}}}
+    hg = {"type": "hgrn2", "mixer": {"heads": nh, "dim": hd, "vdim": hd}, "mlp": None}
+    pa = {"type": "parallel",
+          "mixer": {"left": {"heads": nh, "kv_heads": max(1, nh // 4), "dim": hd, "vdim": hd,
+                             "mask": {"size": 1024}, "rot": {"base": 10000.0, "dims": 64},
+                             "scale": hd ** -0.5},
+                    "right": {"heads": nh, "kv_heads": max(1, nh // 2), "dim": hd, "vdim": hd,
+                              "conv": 4},
+                    "left_scale": 1.0, "right_scale": 1.0},
+          "mlp": {"kind": "dense", "ff": 4 * width}}
+    return HybridConfig.from_dict(
+        {"architecture": "Rotutar", "width": width, "vocab": 32000,
+         "norm": {"eps": 1e-5, "groups": 4}, "logit_softcap": 30.0,
+         "layers": [hg, dict(hg, mlp=moe), hg, pa] * 4}, name="rotutar-w%d" % width)
 
 
 def n_params(cfg) -> int:
@@ -91,13 +119,19 @@ def run(a):
     torch.cuda.set_device(dev)
     prompt, batch, ctx, new = a.hybrid_prompt, a.hybrid_batch, a.hybrid_ctx, a.new_tokens
     pages = max(prompt // 64 + 4, batch * ((ctx + new) // 64 + 2)) + 8
+    design = getattr(a, "hybrid_design", "regesun")
     for width in [int(w) for w in a.hybrid_sizes.split(",")]:
         hcfg = regesun_config(width)
         params = n_params(hcfg)
         lcfg = llama_like(width, hcfg.n_layers, params)
-        for cfg in (hcfg, lcfg):
-            hybrid = cfg is hcfg
+        todo = {"regesun": (hcfg, lcfg), "rotutar": (rotutar_config(width), hcfg),
+                "both": (rotutar_config(width), hcfg, lcfg)}[design]
+        for cfg in todo:
+            if getattr(a, "hybrid_only", None) and a.hybrid_only not in cfg.name:
+                continue
+            hybrid = cfg is not lcfg
             if hybrid:
+                params = n_params(cfg)
                 eng = registry.make_engine(cfg, None, dev, kv_pages=pages, max_batch=batch,
                                            max_prefill_tokens=prompt, seed=1)
             else:

@@ -50,12 +50,31 @@ group_route_k(const T* __restrict__ h, int ldh, const float* __restrict__ wr, in
   const int r = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   for (int i = threadIdx.x; i < W; i += blockDim.x) sh[i] = ldf(h, (size_t)r * ldh + i);
   __syncthreads();
-  for (int e = wave; e < E; e += nw) {
-    const float* w = wr + (size_t)e * W;
-    float d = 0.0f;
-    for (int i = lane; i < W; i += 64) d += sh[i] * w[i];
-    d = wave_sum(d);
-    if (lane == 0) ss[e] = sigmoidf_(d);
+  // four experts at a time per wavefront: their weight loads are independent and go out together
+  for (int e0 = wave * 4; e0 < E; e0 += nw * 4) {
+    const float* w0 = wr + (size_t)e0 * W;
+    const float* w1 = wr + (size_t)min(e0 + 1, E - 1) * W;
+    const float* w2 = wr + (size_t)min(e0 + 2, E - 1) * W;
+    const float* w3 = wr + (size_t)min(e0 + 3, E - 1) * W;
+    float d0 = 0.0f, d1 = 0.0f, d2 = 0.0f, d3 = 0.0f;
+#pragma unroll 4
+    for (int i = lane; i < W; i += 64) {
+      float x = sh[i];
+      d0 += x * w0[i];
+      d1 += x * w1[i];
+      d2 += x * w2[i];
+      d3 += x * w3[i];
+    }
+    d0 = wave_sum(d0);
+    d1 = wave_sum(d1);
+    d2 = wave_sum(d2);
+    d3 = wave_sum(d3);
+    if (lane == 0) {
+      ss[e0] = sigmoidf_(d0);
+      if (e0 + 1 < E) ss[e0 + 1] = sigmoidf_(d1);
+      if (e0 + 2 < E) ss[e0 + 2] = sigmoidf_(d2);
+      if (e0 + 3 < E) ss[e0 + 3] = sigmoidf_(d3);
+    }
   }
   __syncthreads();
   if (wave != 0) return;
@@ -158,6 +177,86 @@ expert_gemm_mfma_k(const bf16* __restrict__ x, int ldx, int x_div, const bf16* _
   }
 }
 
+// Many slots per expert (prompts): a block of 2 x 2 wavefronts takes 128 slots x 128 columns;
+// each wavefront owns 64 x 64 (4 x 4 MFMA tiles), so a K step of 32 needs four A and four B
+// fragments for sixteen products; the next step's fragments are loaded while the current
+// products run.  16-slot tiles beyond the expert's count are skipped.
+__global__ void __launch_bounds__(256)
+expert_gemm_mfma_big_k(const bf16* __restrict__ x, int ldx, int x_div, const bf16* __restrict__ w,
+                       const int* __restrict__ cnt, const int* __restrict__ rows, int ldr,
+                       bf16* __restrict__ out, int ldo, int N, int K) {
+  const int e = blockIdx.z, c = cnt[e];
+  const int m0 = blockIdx.x * 128, n0 = blockIdx.y * 128;
+  if (m0 >= c) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n16 = lane & 15, quad = lane >> 4;
+  const int mbase = m0 + (wave >> 1) * 64, nbase = n0 + (wave & 1) * 64;
+  const int nmt = min(4, (c - mbase + 15) / 16);
+  if (nmt <= 0 || nbase >= N) return;
+  int slot[4];
+  const bf16* xa[4];
+  const bf16* wb[4];
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    int mi = mbase + t * 16 + n16;
+    slot[t] = mi < c ? rows[(size_t)e * ldr + mi] : -1;
+    xa[t] = slot[t] >= 0 ? x + (size_t)(slot[t] / x_div) * ldx + quad * 8 : nullptr;
+    int n = nbase + t * 16 + n16;
+    wb[t] = n < N ? w + ((size_t)e * N + n) * K + quad * 8 : nullptr;
+  }
+  f32x4 acc[4][4];
+#pragma unroll
+  for (int a = 0; a < 4; a++)
+#pragma unroll
+    for (int b = 0; b < 4; b++) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  uint4 af[4], bfr[4];
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  bool kin = quad * 8 < K;
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    af[t] = (xa[t] && kin) ? *(const uint4*)xa[t] : zero;
+    bfr[t] = (wb[t] && kin) ? *(const uint4*)wb[t] : zero;
+  }
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    uint4 an[4], bn[4];
+    const int kn = k0 + 32;
+    const bool nin = kn + quad * 8 < K;
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      an[t] = (xa[t] && nin && t < nmt) ? *(const uint4*)(xa[t] + kn) : zero;
+      bn[t] = (wb[t] && nin) ? *(const uint4*)(wb[t] + kn) : zero;
+    }
+#pragma unroll
+    for (int a = 0; a < 4; a++) {
+      if (a < nmt) {
+        bf16x8 av = __builtin_bit_cast(bf16x8, af[a]);
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, __builtin_bit_cast(bf16x8, bfr[b]),
+                                                               acc[a][b], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      af[t] = an[t];
+      bfr[t] = bn[t];
+    }
+  }
+#pragma unroll
+  for (int a = 0; a < 4; a++) {
+    if (a >= nmt) continue;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      int so = __shfl(slot[a], quad * 4 + i, 64);
+      if (so < 0) continue;
+#pragma unroll
+      for (int b = 0; b < 4; b++) {
+        int n = nbase + b * 16 + n16;
+        if (n < N) out[(size_t)so * ldo + n] = __float2bfloat16(acc[a][b][i]);
+      }
+    }
+  }
+}
+
 // any type, any shape: 32 slots x 64 columns per block, K staged through LDS 32 at a time
 #define EG_KT 32
 template <typename T>
@@ -251,6 +350,12 @@ int p2p_sm_expert_gemm(const void* x, int ldx, int x_div, const void* w, const i
   if (max_slots <= 0 || E <= 0) return 0;
   if (x_div < 1 || N < 1 || K < 1) return (int)hipErrorInvalidValue;
   if (!f32 && K % 8 == 0 && ldx % 8 == 0 && ((size_t)x & 15) == 0 && ((size_t)w & 15) == 0) {
+    if (max_slots >= 512) {   // prompts: the large tile
+      dim3 grid((max_slots + 127) / 128, (N + 127) / 128, E);
+      hipLaunchKernelGGL(expert_gemm_mfma_big_k, grid, dim3(256), 0, st, (const bf16*)x, ldx, x_div,
+                         (const bf16*)w, cnt, rows, ldr, (bf16*)out, ldo, N, K);
+      return (int)hipGetLastError();
+    }
     dim3 grid((max_slots + 63) / 64, (N + 63) / 64, E);
     hipLaunchKernelGGL(expert_gemm_mfma_k, grid, dim3(256), 0, st, (const bf16*)x, ldx, x_div,
                        (const bf16*)w, cnt, rows, ldr, (bf16*)out, ldo, N, K);

@@ -15,6 +15,15 @@
 // staging: HGRN2's silu(q) and f = lower + (1 - lower) sigmoid(. + b); the delta rule's unit q
 // and k (x / sqrt(|x|^2 + 1e-6), q also times D^-1/2), beta = sigmoid(.) and the decay
 // g = exp(-exp(A_log_h) softplus(. + dt_bias)).
+//
+// Long portions run as chunks side by side (the recurrences are linear in the state):
+//   local pass   every chunk from a zero state; its end state, and what carries a state across
+//                the chunk: the product of its decays per key channel (plain write) or the
+//                D x D transition obtained by running the recurrence without values on the
+//                identity (delta rule);
+//   chain        init_{c+1} = T_c init_c + local_c over each portion's chunks, from the slot's
+//                state (or zero at position 0); the last one is the slot's new state;
+//   output pass  every chunk again from its true initial state, with the outputs.
 #include "common.h"
 using namespace sm;
 
@@ -32,27 +41,38 @@ struct ScanArgs {
   const float* normw; float* state; const int* ent; void* out; int ldo;
   int H, G, D, V, CT;
   float eps, out_scale;
+  // 0: portions from their slots' states, states written back.  Chunk modes (`ent` lists chunks,
+  // its slot field is the chunk index into the buffers below): 1: from zero, end state ->
+  // chunk_state (and the decay product -> chunk_decay for the plain write); 2: from
+  // chunk_state, outputs only; 3 (delta rule): the transition on the identity -> chunk_trans.
+  int mode;
+  float* chunk_state;   // [chunks, H, D, V]
+  float* chunk_decay;   // [chunks, H, D]
+  float* chunk_trans;   // [chunks, H, D, D]
 };
 
 template <typename T, int DQ, bool DELTA>
 __global__ void __launch_bounds__(1024) gated_scan_k(ScanArgs a) {
   constexpr int DKP = 4 * DQ;   // padded key index (zero filled in LDS)
-  const int H = a.H, D = a.D, V = a.V, CT = a.CT;
+  const int H = a.H, D = a.D, V = a.V, CT = a.CT, mode = a.mode;
   const int e = blockIdx.x / H, h = blockIdx.x % H;
   const Entry en = load_entry(a.ent, e);
   if (en.n <= 0) return;
+  const bool trans = mode == 3;
+  const int NC = trans ? D : V;                // columns of the matrix this block carries
   const int nw = blockDim.x >> 6, VP = nw * 16;
-  extern __shared__ float smem[];
+  extern __shared__ __align__(16) float smem[];
   float* sq = smem;                  // [CT][DKP]
   float* sk = sq + CT * DKP;
   float* sg = sk + CT * DKP;
   float* sv = sg + CT * DKP;         // [CT][VP]
   float* so = sv + CT * VP;          // [CT][VP]
   float* sb = so + CT * VP;          // [CT]
+  float* sP = sb + CT;               // [DKP] product of the chunk's decays (mode 1, plain write)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int j = wave * 16 + (lane & 15), is = lane >> 4, i0 = is * DQ;
-  const bool act = j < V;
-  const int jc = min(j, V - 1);
+  const bool act = j < NC;
+  const int jc = min(j, NC - 1);
   const int hk = DELTA ? h / (H / a.G) : h;    // the q/k head this head reads
   const T* proj = (const T*)a.proj;
   const T* araw = (const T*)a.araw;
@@ -60,13 +80,19 @@ __global__ void __launch_bounds__(1024) gated_scan_k(ScanArgs a) {
   const T* gate = (const T*)a.gate;
   T* out = (T*)a.out;
   float S[DQ];
-  float* Sg = a.state + ((size_t)en.slot * H + h) * D * V;
+  float* Sg = mode == 0 ? a.state + ((size_t)en.slot * H + h) * D * V
+            : trans     ? a.chunk_trans + ((size_t)en.slot * H + h) * D * D
+                        : a.chunk_state + ((size_t)en.slot * H + h) * D * V;
+  const bool from_state = mode == 2 || (mode == 0 && en.start > 0);
 #pragma unroll
   for (int q = 0; q < DQ; q++) {
     // loads at clamped addresses, selected afterwards, so that they go out together
-    float vv = en.start > 0 ? Sg[(size_t)min(i0 + q, D - 1) * V + jc] : 0.0f;
+    float v0 = (trans && i0 + q == j) ? 1.0f : 0.0f;
+    float vv = from_state ? Sg[(size_t)min(i0 + q, D - 1) * NC + jc] : v0;
     S[q] = (act && i0 + q < D) ? vv : 0.0f;
   }
+  if (!DELTA && mode == 1)
+    for (int i = threadIdx.x; i < DKP; i += blockDim.x) sP[i] = 1.0f;
   const float negA = DELTA ? -expf(a.A_log[h]) : 0.0f;
   const float qscale = DELTA ? 1.0f / sqrtf((float)D) : 1.0f;
   for (int t0 = 0; t0 < en.n; t0 += CT) {
@@ -91,14 +117,15 @@ __global__ void __launch_bounds__(1024) gated_scan_k(ScanArgs a) {
       }
       sq[idx] = vq; sk[idx] = vk; sg[idx] = vg;
     }
-    for (int idx = threadIdx.x; idx < ct * VP; idx += blockDim.x) {
-      int t = idx / VP, i = idx % VP;
-      size_t row = (size_t)(en.row0 + t0 + t);
-      float vv = 0.0f;
-      if (i < V) vv = DELTA ? a.conv[row * a.ldc + 2 * a.G * D + h * V + i]
-                            : ldf(proj, row * a.ldp + 2 * H * D + h * V + i);
-      sv[idx] = vv;
-    }
+    if (!trans)
+      for (int idx = threadIdx.x; idx < ct * VP; idx += blockDim.x) {
+        int t = idx / VP, i = idx % VP;
+        size_t row = (size_t)(en.row0 + t0 + t);
+        float vv = 0.0f;
+        if (i < V) vv = DELTA ? a.conv[row * a.ldc + 2 * a.G * D + h * V + i]
+                              : ldf(proj, row * a.ldp + 2 * H * D + h * V + i);
+        sv[idx] = vv;
+      }
     if (DELTA) {
       for (int t = threadIdx.x; t < ct; t += blockDim.x)
         sb[t] = sigmoidf_(ldf(braw, (size_t)(en.row0 + t0 + t) * a.ldb + h));
@@ -121,36 +148,54 @@ __global__ void __launch_bounds__(1024) gated_scan_k(ScanArgs a) {
       }
     }
     __syncthreads();
+    if (!DELTA && mode == 1)
+      for (int i = threadIdx.x; i < D; i += blockDim.x) {
+        float p = sP[i];
+        for (int t = 0; t < ct; t++) p *= sg[t * DKP + i];
+        sP[i] = p;
+      }
     for (int t = 0; t < ct; t++) {   // every lane takes part (the shuffles need all of them)
-      const float* kr = sk + t * DKP + i0;
-      const float* gr = sg + t * DKP + i0;
-      const float* qr = sq + t * DKP + i0;
-      float u = sv[t * VP + jc];
+      const float4* k4 = (const float4*)(sk + t * DKP + i0);
+      const float4* g4 = (const float4*)(sg + t * DKP + i0);
+      const float4* q4 = (const float4*)(sq + t * DKP + i0);
+      float u = trans ? 0.0f : sv[t * VP + jc];
       if (DELTA) {
-        float d = 0.0f;
+        float d0 = 0.0f, d1 = 0.0f, d2 = 0.0f, d3 = 0.0f;   // four chains instead of one
 #pragma unroll
-        for (int q = 0; q < DQ; q++) {
-          S[q] *= gr[q];
-          d += kr[q] * S[q];
+        for (int q = 0; q < DQ / 4; q++) {
+          float4 g = g4[q], k = k4[q];
+          S[4 * q] *= g.x; S[4 * q + 1] *= g.y; S[4 * q + 2] *= g.z; S[4 * q + 3] *= g.w;
+          d0 += k.x * S[4 * q]; d1 += k.y * S[4 * q + 1];
+          d2 += k.z * S[4 * q + 2]; d3 += k.w * S[4 * q + 3];
         }
+        float d = (d0 + d1) + (d2 + d3);
         d += __shfl_xor(d, 16, 64);
         d += __shfl_xor(d, 32, 64);
         u = sb[t] * (u - d);
       } else {
 #pragma unroll
-        for (int q = 0; q < DQ; q++) S[q] *= gr[q];
+        for (int q = 0; q < DQ / 4; q++) {
+          float4 g = g4[q];
+          S[4 * q] *= g.x; S[4 * q + 1] *= g.y; S[4 * q + 2] *= g.z; S[4 * q + 3] *= g.w;
+        }
       }
-      float o = 0.0f;
+      float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
 #pragma unroll
-      for (int q = 0; q < DQ; q++) {
-        S[q] += kr[q] * u;
-        o += S[q] * qr[q];
+      for (int q = 0; q < DQ / 4; q++) {
+        float4 k = k4[q], qv = q4[q];
+        S[4 * q] += k.x * u; S[4 * q + 1] += k.y * u; S[4 * q + 2] += k.z * u; S[4 * q + 3] += k.w * u;
+        o0 += S[4 * q] * qv.x; o1 += S[4 * q + 1] * qv.y;
+        o2 += S[4 * q + 2] * qv.z; o3 += S[4 * q + 3] * qv.w;
       }
-      o += __shfl_xor(o, 16, 64);
-      o += __shfl_xor(o, 32, 64);
-      if (is == 0) so[t * VP + j] = act ? o : 0.0f;
+      if (mode == 0 || mode == 2) {
+        float o = (o0 + o1) + (o2 + o3);
+        o += __shfl_xor(o, 16, 64);
+        o += __shfl_xor(o, 32, 64);
+        if (is == 0) so[t * VP + j] = act ? o : 0.0f;
+      }
     }
     __syncthreads();
+    if (mode == 0 || mode == 2)
     for (int t = wave; t < ct; t += nw) {
       float ss = 0.0f;
       for (int i = lane; i < V; i += 64) ss += so[t * VP + i] * so[t * VP + i];
@@ -167,11 +212,88 @@ __global__ void __launch_bounds__(1024) gated_scan_k(ScanArgs a) {
     // written again only after the next staging barrier, which every wave reaches after its
     // share of this chunk's outputs
   }
-  if (act) {
+  if (act && mode != 2) {
 #pragma unroll
     for (int q = 0; q < DQ; q++)
-      if (i0 + q < D) Sg[(size_t)(i0 + q) * V + j] = S[q];
+      if (i0 + q < D) Sg[(size_t)(i0 + q) * NC + j] = S[q];
   }
+  if (!DELTA && mode == 1) {
+    __syncthreads();
+    for (int i = threadIdx.x; i < D; i += blockDim.x)
+      a.chunk_decay[((size_t)en.slot * H + h) * D + i] = sP[i];
+  }
+}
+
+// Chain of the plain write: the transition of a chunk is diagonal.  One thread per state
+// element walks its portion's chunks: init_c replaces local_c in `cs`, the end goes to the slot.
+__global__ void __launch_bounds__(256)
+diag_chain_k(float* __restrict__ cs, const float* __restrict__ decay, float* __restrict__ state,
+             const int* __restrict__ cent, int H, int D, int V) {
+  const int e = blockIdx.y / H, h = blockIdx.y % H;
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= D * V) return;
+  const int i = idx / V;
+  const int c0 = cent[4 * e], nc = cent[4 * e + 1], start = cent[4 * e + 2], slot = cent[4 * e + 3];
+  float* sg = state + ((size_t)slot * H + h) * D * V + idx;
+  float cur = start > 0 ? *sg : 0.0f;
+  for (int c = c0; c < c0 + nc; c++) {
+    float* p = cs + ((size_t)c * H + h) * D * V + idx;
+    float local = *p;
+    *p = cur;
+    cur = decay[((size_t)c * H + h) * D + i] * cur + local;
+  }
+  *sg = cur;
+}
+
+// Chain of the delta rule: init_{c+1} = T_c . init_c + local_c with a dense D x D transition.
+// The columns of the state are independent: one block per (portion, head, 16 columns), the
+// current columns in LDS, thread (column, row group) forms every 16th row of the product.
+#define DC_ROWS 16   // rows per thread at most (D <= 256)
+__global__ void __launch_bounds__(256)
+dense_chain_k(float* __restrict__ cs, const float* __restrict__ trans, float* __restrict__ state,
+              const int* __restrict__ cent, int H, int D, int V) {
+  extern __shared__ float scur[];   // [D][17]
+  const int e = blockIdx.y / H, h = blockIdx.y % H;
+  const int col = threadIdx.x & 15, rg = threadIdx.x >> 4;
+  const int j = blockIdx.x * 16 + col;
+  const bool act = j < V;
+  const int jc = min(j, V - 1);
+  const int c0 = cent[4 * e], nc = cent[4 * e + 1], start = cent[4 * e + 2], slot = cent[4 * e + 3];
+  float* sg = state + ((size_t)slot * H + h) * D * V;
+  for (int i = rg; i < D; i += 16) scur[i * 17 + col] = (start > 0 && act) ? sg[(size_t)i * V + jc] : 0.0f;
+  __syncthreads();
+  for (int c = c0; c < c0 + nc; c++) {
+    float* loc = cs + ((size_t)c * H + h) * D * V;
+    const float* Tc = trans + ((size_t)c * H + h) * D * D;
+    float nv[DC_ROWS];
+#pragma unroll
+    for (int r = 0; r < DC_ROWS; r++) {
+      int i = rg + 16 * r;
+      if (i < D) {
+        float acc0 = loc[(size_t)i * V + jc], acc1 = 0.0f;
+        const float* Ti = Tc + (size_t)i * D;
+        int k = 0;
+        for (; k + 3 < D; k += 4) {
+          acc0 += Ti[k] * scur[k * 17 + col] + Ti[k + 2] * scur[(k + 2) * 17 + col];
+          acc1 += Ti[k + 1] * scur[(k + 1) * 17 + col] + Ti[k + 3] * scur[(k + 3) * 17 + col];
+        }
+        for (; k < D; k++) acc0 += Ti[k] * scur[k * 17 + col];
+        nv[r] = acc0 + acc1;
+      }
+    }
+    __syncthreads();   // every thread has read the old columns
+#pragma unroll
+    for (int r = 0; r < DC_ROWS; r++) {
+      int i = rg + 16 * r;
+      if (i < D) {
+        if (act) loc[(size_t)i * V + j] = scur[i * 17 + col];   // init_c replaces local_c
+        scur[i * 17 + col] = nv[r];
+      }
+    }
+    __syncthreads();
+  }
+  if (act)
+    for (int i = rg; i < D; i += 16) sg[(size_t)i * V + j] = scur[i * 17 + col];
 }
 
 template <bool DELTA>
@@ -179,13 +301,14 @@ static int launch_scan(ScanArgs a, int E, int f32, hipStream_t st) {
   if (E <= 0) return 0;
   if (a.H < 1 || a.D < 1 || a.V < 1 || a.D > 256 || a.V > 256 || a.G < 1 || a.H % a.G)
     return (int)hipErrorInvalidValue;
-  int nw = (a.V + 15) / 16;
+  int cols = a.mode == 3 ? a.D : a.V;
+  int nw = (cols + 15) / 16;
   int dq = a.D <= 32 ? 8 : a.D <= 64 ? 16 : a.D <= 128 ? 32 : 64;
   int per_tok = 3 * 4 * dq + 2 * nw * 16 + 1;
   int CT = 16;
-  while (CT > 2 && (size_t)CT * per_tok * 4 > 48 * 1024) CT /= 2;
+  while (CT > 2 && (size_t)(CT * per_tok + 4 * dq) * 4 > 48 * 1024) CT /= 2;
   a.CT = CT;
-  size_t shm = (size_t)CT * per_tok * 4;
+  size_t shm = (size_t)(CT * per_tok + 4 * dq) * 4;
   dim3 grid(E * a.H), block(64 * nw);
 #define GS(DQ)                                                                              \
   SM_DISPATCH_T(f32, hipLaunchKernelGGL((gated_scan_k<T, DQ, DELTA>), grid, block, shm, st, a))
@@ -195,6 +318,32 @@ static int launch_scan(ScanArgs a, int E, int f32, hipStream_t st) {
   else GS(64);
 #undef GS
   return (int)hipGetLastError();
+}
+
+// the three passes over `NV` chunks (vent) of `E` portions (cent = first chunk, chunks, first
+// position, slot); cs [NV, H, D, V], cd [NV, H, D] (plain write) or ct [NV, H, D, D] (delta rule)
+template <bool DELTA>
+static int launch_chunked(ScanArgs a, const int* vent, int NV, const int* cent, int E, float* cs,
+                          float* cd, float* ct, int f32, hipStream_t st) {
+  if (NV <= 0 || E <= 0) return 0;
+  float* state = a.state;
+  a.ent = vent;
+  a.chunk_state = cs; a.chunk_decay = cd; a.chunk_trans = ct;
+  a.mode = 1;
+  int err = launch_scan<DELTA>(a, NV, f32, st);
+  if (err) return err;
+  if (DELTA) {
+    a.mode = 3;
+    if ((err = launch_scan<DELTA>(a, NV, f32, st))) return err;
+    hipLaunchKernelGGL(dense_chain_k, dim3((a.V + 15) / 16, E * a.H), dim3(256),
+                       (size_t)a.D * 17 * 4, st, cs, ct, state, cent, a.H, a.D, a.V);
+  } else {
+    hipLaunchKernelGGL(diag_chain_k, dim3((a.D * a.V + 255) / 256, E * a.H), dim3(256), 0, st, cs,
+                       cd, state, cent, a.H, a.D, a.V);
+  }
+  if ((err = (int)hipGetLastError())) return err;
+  a.mode = 2;
+  return launch_scan<DELTA>(a, NV, f32, st);
 }
 
 extern "C" {
@@ -220,6 +369,33 @@ int p2p_sm_gated_delta_scan(const float* conv, int ldc, const void* araw, int ld
   a.normw = normw; a.state = state; a.ent = ent; a.out = out; a.ldo = ldo;
   a.H = H; a.G = G; a.D = D; a.V = V; a.eps = eps; a.out_scale = out_scale;
   return launch_scan<true>(a, E, f32, st);
+}
+
+int p2p_sm_hgrn2_scan_chunked(const void* proj, int ldp, const float* lower, const float* fb,
+                              const float* normw, float* state, float* cs, float* cd,
+                              const int* vent, int NV, const int* cent, int E, void* out, int ldo,
+                              int H, int D, int V, float eps, float out_scale, int f32,
+                              hipStream_t st) {
+  ScanArgs a = {};
+  a.proj = proj; a.ldp = ldp; a.lower = lower; a.fb = fb;
+  a.normw = normw; a.state = state; a.out = out; a.ldo = ldo;
+  a.H = H; a.G = H; a.D = D; a.V = V; a.eps = eps; a.out_scale = out_scale;
+  return launch_chunked<false>(a, vent, NV, cent, E, cs, cd, nullptr, f32, st);
+}
+
+int p2p_sm_gated_delta_scan_chunked(const float* conv, int ldc, const void* araw, int lda,
+                                    const void* braw, int ldb, const void* gate, int ldg,
+                                    const float* A_log, const float* dt_bias, const float* normw,
+                                    float* state, float* cs, float* ct, const int* vent, int NV,
+                                    const int* cent, int E, void* out, int ldo, int H, int G,
+                                    int D, int V, float eps, float out_scale, int f32,
+                                    hipStream_t st) {
+  ScanArgs a = {};
+  a.conv = conv; a.ldc = ldc; a.araw = araw; a.lda = lda; a.braw = braw; a.ldb = ldb;
+  a.gate = gate; a.ldg = ldg; a.A_log = A_log; a.dt_bias = dt_bias;
+  a.normw = normw; a.state = state; a.out = out; a.ldo = ldo;
+  a.H = H; a.G = G; a.D = D; a.V = V; a.eps = eps; a.out_scale = out_scale;
+  return launch_chunked<true>(a, vent, NV, cent, E, cs, nullptr, ct, f32, st);
 }
 
 }  // extern "C"

@@ -81,6 +81,14 @@ _SIGS = {
     "p2p_sm_hgrn2_scan": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_int, c_void_p, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
                           c_void_p],
+    "p2p_sm_hgrn2_scan_chunked": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                  c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
+                                  c_int, c_int, c_int, c_float, c_float, c_int, c_void_p],
+    "p2p_sm_gated_delta_scan_chunked": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p,
+                                        c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                        c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p,
+                                        c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
+                                        c_void_p],
     "p2p_sm_gated_delta_scan": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p,
                                 c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                 c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float,
@@ -842,6 +850,17 @@ def hgrn2_scan(proj, lower, fb, normw, state, ent, ent_host, out, H: int, D: int
     _vec(fb, n, "fb")
     _vec(normw, V, "normw")
     _scan_state_ok(state, H, D, V, ent)
+    if _chunked(ent_host):
+        vent, cent = (t_.to(proj.device) for t_ in scan_chunks(ent_host, SCAN_CHUNK))
+        NV = vent.shape[0]
+        cs = torch.empty(NV, H, D, V, device=proj.device, dtype=torch.float32)
+        cd = torch.empty(NV, H, D, device=proj.device, dtype=torch.float32)
+        _chk(lib().p2p_sm_hgrn2_scan_chunked(
+            proj.data_ptr(), proj.stride(0), lower.data_ptr(), fb.data_ptr(), normw.data_ptr(),
+            state.data_ptr(), cs.data_ptr(), cd.data_ptr(), vent.data_ptr(), NV, cent.data_ptr(),
+            ent.shape[0], out.data_ptr(), out.stride(0), H, D, V, eps, out_scale, _f32(proj),
+            _st(proj)), "hgrn2_scan_chunked")
+        return out
     _chk(lib().p2p_sm_hgrn2_scan(proj.data_ptr(), proj.stride(0), lower.data_ptr(), fb.data_ptr(),
                                  normw.data_ptr(), state.data_ptr(), ent.data_ptr(), ent.shape[0],
                                  out.data_ptr(), out.stride(0), H, D, V, eps, out_scale,
@@ -896,6 +915,18 @@ def gated_delta_scan(conv, araw, braw, gate, A_log, dt_bias, normw, state, ent, 
     _vec(normw, V, "normw")
     assert H % G == 0
     _scan_state_ok(state, H, D, V, ent)
+    if _chunked(ent_host):
+        vent, cent = (t_.to(conv.device) for t_ in scan_chunks(ent_host, SCAN_CHUNK))
+        NV = vent.shape[0]
+        cs = torch.empty(NV, H, D, V, device=conv.device, dtype=torch.float32)
+        ct = torch.empty(NV, H, D, D, device=conv.device, dtype=torch.float32)
+        _chk(lib().p2p_sm_gated_delta_scan_chunked(
+            conv.data_ptr(), conv.stride(0), araw.data_ptr(), araw.stride(0), braw.data_ptr(),
+            braw.stride(0), gate.data_ptr(), gate.stride(0), A_log.data_ptr(), dt_bias.data_ptr(),
+            normw.data_ptr(), state.data_ptr(), cs.data_ptr(), ct.data_ptr(), vent.data_ptr(), NV,
+            cent.data_ptr(), ent.shape[0], out.data_ptr(), out.stride(0), H, G, D, V, eps,
+            out_scale, _f32(out), _st(out)), "gated_delta_scan_chunked")
+        return out
     _chk(lib().p2p_sm_gated_delta_scan(conv.data_ptr(), conv.stride(0), araw.data_ptr(),
                                        araw.stride(0), braw.data_ptr(), braw.stride(0),
                                        gate.data_ptr(), gate.stride(0), A_log.data_ptr(),
