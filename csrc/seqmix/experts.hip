@@ -9,10 +9,9 @@
 //
 // expert_gemm: for expert e and each of its slots s: out[s] = x[s / x_div] . W_e^T.  Rows are
 // gathered through the slot lists, so only experts with rows read their weights.  bf16 runs
-// on the matrix cores (operands straight from global memory into MFMA fragments: the A rows
-// are gathered anyway and the weights of an expert are shared through L2 by the blocks that
-// work on it); fp32 and odd shapes run a tiled FMA kernel.  A slot's result does not depend on
-// which other slots share its tile.
+// on the matrix cores (a 16 x 64 tile with K split over the wavefronts for decode-sized steps,
+// an LDS-staged 128 x 128 tile for prompts); fp32 and odd shapes run a tiled FMA kernel.  A
+// slot's result does not depend on which other slots share its tile.
 #include "common.h"
 using namespace sm;
 
@@ -126,45 +125,122 @@ group_route_k(const T* __restrict__ h, int ldh, const float* __restrict__ wr, in
   }
 }
 
-// bf16 on the matrix cores: a block of 4 wavefronts takes 64 slots x 64 output columns of one
-// expert; wavefront w owns 16 slots and walks K in steps of 32 with one A fragment (its
-// gathered rows) and four B fragments (16 weight rows each) per step.
+// The grid is sized for the most row tiles the experts can have together (total slots / BM + E,
+// since every expert wastes at most one partial tile), one-dimensional, and workgroups go to
+// the 8 XCDs round-robin: block L runs on XCD L % 8.  A block counts the row tiles that exist,
+// deals them to the XCDs in contiguous runs of equal length (XCD j takes row tiles
+// j*pr .. j*pr+pr-1 and all column tiles, so its L2 holds the gathered rows of few experts and
+// streams only those experts' weights), and finds its expert and first slot by walking the
+// counts.  Blocks beyond the tiles that exist leave at once.
+__device__ __forceinline__ bool find_tile(const int* __restrict__ cnt, int E, int BM,
+                                          int row_tiles_pad, int& e, int& m0, int& nt) {
+  // every wavefront does this for itself, 64 experts at a time: one vector load of the counts,
+  // sums and prefix sums by lane shuffles (a scalar walk over the counts costs a dependent
+  // load per expert, which a decode-sized launch cannot hide)
+  const int lane = threadIdx.x & 63;
+  int total = 0;
+  for (int base = 0; base < E; base += 64) {
+    int i = base + lane;
+    int n = i < E ? (cnt[i] + BM - 1) / BM : 0;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) n += __shfl_xor(n, o, 64);
+    total += n;
+  }
+  const int j = blockIdx.x & 7, s = blockIdx.x >> 3, pm = row_tiles_pad >> 3;
+  const int pr = (total + 7) >> 3, li = s % pm;
+  nt = s / pm;
+  const int t = j * pr + li;
+  if (li >= pr || t >= total) return false;
+  int acc = 0, fe = -1, fm = 0;
+  for (int base = 0; base < E && fe < 0; base += 64) {
+    int i = base + lane;
+    int n = i < E ? (cnt[i] + BM - 1) / BM : 0;
+    int incl = n;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      int v = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += v;
+    }
+    int excl = acc + incl - n;
+    bool hit = n > 0 && t >= excl && t < excl + n;
+    unsigned long long mask = __ballot(hit);
+    if (mask) {
+      int src = __ffsll((long long)mask) - 1;
+      fe = base + src;
+      fm = (t - __shfl(excl, src, 64)) * BM;
+    }
+    acc += __shfl(incl, 63, 64);
+  }
+  // the same for every lane: keep them in scalar registers
+  e = __builtin_amdgcn_readfirstlane(fe);
+  m0 = __builtin_amdgcn_readfirstlane(fm);
+  return e >= 0;
+}
+
+// bf16 on the matrix cores, few slots per expert (decode-sized steps): a block takes 16 slots x
+// 64 output columns of one expert and its four wavefronts split K among themselves, so the
+// chain of dependent loads is a quarter as long; each wavefront walks its share in steps of 32
+// with one A fragment (the gathered rows) and four B fragments (16 weight rows each), the next
+// step's fragments in flight while the current products run; the four partial tiles are
+// added through LDS.
 __global__ void __launch_bounds__(256)
 expert_gemm_mfma_k(const bf16* __restrict__ x, int ldx, int x_div, const bf16* __restrict__ w,
                    const int* __restrict__ cnt, const int* __restrict__ rows, int ldr,
-                   bf16* __restrict__ out, int ldo, int N, int K) {
-  const int e = blockIdx.z, c = cnt[e];
-  const int m0 = blockIdx.x * 64, n0 = blockIdx.y * 64;
-  if (m0 >= c) return;
+                   bf16* __restrict__ out, int ldo, int N, int K, int E, int TMP) {
+  __shared__ f32x4 red[3][4][64];
+  int e, m0, nt;
+  if (!find_tile(cnt, E, 16, TMP, e, m0, nt)) return;
+  const int c = cnt[e], n0 = nt * 64;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n16 = lane & 15, quad = lane >> 4;
-  const int mi = m0 + wave * 16 + n16;
+  const int mi = m0 + n16;
   const int slot = mi < c ? rows[(size_t)e * ldr + mi] : -1;
-  if (m0 + wave * 16 >= c) return;
-  const bf16* xa = slot >= 0 ? x + (size_t)(slot / x_div) * ldx : nullptr;
+  const int kq = ((K + 127) / 128) * 32;          // K per wavefront, a multiple of 32
+  const int kb = wave * kq, ke = min(K, kb + kq);
+  const bf16* xa = slot >= 0 ? x + (size_t)(slot / x_div) * ldx + quad * 8 : nullptr;
   const bf16* wb[4];
 #pragma unroll
   for (int t = 0; t < 4; t++) {
     int n = n0 + t * 16 + n16;
-    wb[t] = n < N ? w + ((size_t)e * N + n) * K : nullptr;
+    wb[t] = n < N ? w + ((size_t)e * N + n) * K + quad * 8 : nullptr;
   }
   f32x4 acc[4];
 #pragma unroll
   for (int t = 0; t < 4; t++) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    int kc = k0 + quad * 8;
-    bool kin = kc < K;                       // K is a multiple of 8
-    uint4 av = (xa && kin) ? *(const uint4*)(xa + kc) : make_uint4(0, 0, 0, 0);
-    uint4 bv[4];
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  uint4 av, bv[4];
+  {
+    bool kin = kb + quad * 8 < ke;                 // K is a multiple of 8
+    av = (xa && kin) ? *(const uint4*)(xa + kb) : zero;
 #pragma unroll
-    for (int t = 0; t < 4; t++)
-      bv[t] = (wb[t] && kin) ? *(const uint4*)(wb[t] + kc) : make_uint4(0, 0, 0, 0);
+    for (int t = 0; t < 4; t++) bv[t] = (wb[t] && kin) ? *(const uint4*)(wb[t] + kb) : zero;
+  }
+  for (int k0 = kb; k0 < ke; k0 += 32) {
+    const int kn = k0 + 32;
+    const bool nin = kn + quad * 8 < ke;
+    uint4 an = (xa && nin) ? *(const uint4*)(xa + kn) : zero;
+    uint4 bn[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) bn[t] = (wb[t] && nin) ? *(const uint4*)(wb[t] + kn) : zero;
     bf16x8 af = __builtin_bit_cast(bf16x8, av);
 #pragma unroll
     for (int t = 0; t < 4; t++)
       acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, __builtin_bit_cast(bf16x8, bv[t]),
                                                         acc[t], 0, 0, 0);
+    av = an;
+#pragma unroll
+    for (int t = 0; t < 4; t++) bv[t] = bn[t];
   }
-  // accumulator layout: row quad*4 + i of the wave's 16 slots, column n16 of each tile
+  if (wave > 0) {
+#pragma unroll
+    for (int t = 0; t < 4; t++) red[wave - 1][t][lane] = acc[t];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int t = 0; t < 4; t++)
+#pragma unroll
+    for (int u = 0; u < 3; u++) acc[t] += red[u][t][lane];
+  // accumulator layout: row quad*4 + i of the 16 slots, column n16 of each tile
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     int so = __shfl(slot, quad * 4 + i, 64);
@@ -177,80 +253,99 @@ expert_gemm_mfma_k(const bf16* __restrict__ x, int ldx, int x_div, const bf16* _
   }
 }
 
-// Many slots per expert (prompts): a block of 2 x 2 wavefronts takes 128 slots x 128 columns;
-// each wavefront owns 64 x 64 (4 x 4 MFMA tiles), so a K step of 32 needs four A and four B
-// fragments for sixteen products; the next step's fragments are loaded while the current
-// products run.  16-slot tiles beyond the expert's count are skipped.
+// Many slots per expert (prompts): a block of 2 x 2 wavefronts takes 128 slots x 128 columns
+// and walks K in steps of 64.  The gathered A rows and the weight rows of a step are loaded
+// with coalesced 16-byte reads (8 threads per row), kept in registers while the previous step
+// computes, and handed to the MFMA fragments through LDS (rows 144 bytes apart).  Each
+// wavefront owns 64 x 64 (4 x 4 MFMA tiles); 16-slot tiles beyond the expert's count are skipped.
+#define EB_LD 72   // bf16 per LDS row: 64 + 8
 __global__ void __launch_bounds__(256)
 expert_gemm_mfma_big_k(const bf16* __restrict__ x, int ldx, int x_div, const bf16* __restrict__ w,
                        const int* __restrict__ cnt, const int* __restrict__ rows, int ldr,
-                       bf16* __restrict__ out, int ldo, int N, int K) {
-  const int e = blockIdx.z, c = cnt[e];
-  const int m0 = blockIdx.x * 128, n0 = blockIdx.y * 128;
-  if (m0 >= c) return;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n16 = lane & 15, quad = lane >> 4;
-  const int mbase = m0 + (wave >> 1) * 64, nbase = n0 + (wave & 1) * 64;
-  const int nmt = min(4, (c - mbase + 15) / 16);
-  if (nmt <= 0 || nbase >= N) return;
-  int slot[4];
-  const bf16* xa[4];
-  const bf16* wb[4];
+                       bf16* __restrict__ out, int ldo, int N, int K, int E, int TMP) {
+  __shared__ __align__(16) unsigned short sA[128 * EB_LD];
+  __shared__ __align__(16) unsigned short sB[128 * EB_LD];
+  __shared__ int sslot[128];
+  int e, m0, nt;
+  if (!find_tile(cnt, E, 128, TMP, e, m0, nt)) return;
+  const int c = cnt[e], n0 = nt * 128;
+  const int tid = threadIdx.x;
+  if (tid < 128) sslot[tid] = m0 + tid < c ? rows[(size_t)e * ldr + m0 + tid] : -1;
+  __syncthreads();
+  const int lane = tid & 63, wave = tid >> 6, n16 = lane & 15, quad = lane >> 4;
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  const int nmt = max(0, min(4, (c - (m0 + wm) + 15) / 16));
+  // this thread's four 16-byte pieces of the A and B tiles: row = (tid + 256 u) / 8
+  const int c8 = (tid & 7) * 8;
+  const bf16* pa[4];
+  const bf16* pb[4];
 #pragma unroll
-  for (int t = 0; t < 4; t++) {
-    int mi = mbase + t * 16 + n16;
-    slot[t] = mi < c ? rows[(size_t)e * ldr + mi] : -1;
-    xa[t] = slot[t] >= 0 ? x + (size_t)(slot[t] / x_div) * ldx + quad * 8 : nullptr;
-    int n = nbase + t * 16 + n16;
-    wb[t] = n < N ? w + ((size_t)e * N + n) * K + quad * 8 : nullptr;
+  for (int u = 0; u < 4; u++) {
+    int r = (tid + 256 * u) >> 3;
+    int sl = sslot[r];
+    pa[u] = sl >= 0 ? x + (size_t)(sl / x_div) * ldx + c8 : nullptr;
+    pb[u] = n0 + r < N ? w + ((size_t)e * N + n0 + r) * K + c8 : nullptr;
+  }
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  uint4 ra[4], rb[4];
+#pragma unroll
+  for (int u = 0; u < 4; u++) {
+    bool kin = c8 < K;
+    ra[u] = (pa[u] && kin) ? *(const uint4*)pa[u] : zero;
+    rb[u] = (pb[u] && kin) ? *(const uint4*)pb[u] : zero;
   }
   f32x4 acc[4][4];
 #pragma unroll
   for (int a = 0; a < 4; a++)
 #pragma unroll
     for (int b = 0; b < 4; b++) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
-  uint4 af[4], bfr[4];
-  const uint4 zero = make_uint4(0, 0, 0, 0);
-  bool kin = quad * 8 < K;
+  for (int k0 = 0; k0 < K; k0 += 64) {
 #pragma unroll
-  for (int t = 0; t < 4; t++) {
-    af[t] = (xa[t] && kin) ? *(const uint4*)xa[t] : zero;
-    bfr[t] = (wb[t] && kin) ? *(const uint4*)wb[t] : zero;
-  }
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    uint4 an[4], bn[4];
-    const int kn = k0 + 32;
-    const bool nin = kn + quad * 8 < K;
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-      an[t] = (xa[t] && nin && t < nmt) ? *(const uint4*)(xa[t] + kn) : zero;
-      bn[t] = (wb[t] && nin) ? *(const uint4*)(wb[t] + kn) : zero;
+    for (int u = 0; u < 4; u++) {
+      int r = (tid + 256 * u) >> 3;
+      *(uint4*)(sA + r * EB_LD + c8) = ra[u];
+      *(uint4*)(sB + r * EB_LD + c8) = rb[u];
     }
+    __syncthreads();
+    const int kn = k0 + 64;
+    if (kn < K) {
+      bool kin = kn + c8 < K;
 #pragma unroll
-    for (int a = 0; a < 4; a++) {
-      if (a < nmt) {
-        bf16x8 av = __builtin_bit_cast(bf16x8, af[a]);
-#pragma unroll
-        for (int b = 0; b < 4; b++)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, __builtin_bit_cast(bf16x8, bfr[b]),
-                                                               acc[a][b], 0, 0, 0);
+      for (int u = 0; u < 4; u++) {
+        ra[u] = (pa[u] && kin) ? *(const uint4*)(pa[u] + kn) : zero;
+        rb[u] = (pb[u] && kin) ? *(const uint4*)(pb[u] + kn) : zero;
       }
     }
 #pragma unroll
-    for (int t = 0; t < 4; t++) {
-      af[t] = an[t];
-      bfr[t] = bn[t];
+    for (int kk = 0; kk < 2; kk++) {
+      bf16x8 bfr[4];
+#pragma unroll
+      for (int b = 0; b < 4; b++)
+        bfr[b] = __builtin_bit_cast(bf16x8, *(const uint4*)(sB + (wn + b * 16 + n16) * EB_LD +
+                                                             kk * 32 + quad * 8));
+#pragma unroll
+      for (int a = 0; a < 4; a++) {
+        if (a < nmt) {
+          bf16x8 av = __builtin_bit_cast(bf16x8, *(const uint4*)(sA + (wm + a * 16 + n16) * EB_LD +
+                                                                  kk * 32 + quad * 8));
+#pragma unroll
+          for (int b = 0; b < 4; b++)
+            acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bfr[b], acc[a][b], 0, 0, 0);
+        }
+      }
     }
+    __syncthreads();
   }
 #pragma unroll
   for (int a = 0; a < 4; a++) {
     if (a >= nmt) continue;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      int so = __shfl(slot[a], quad * 4 + i, 64);
+      int so = sslot[wm + a * 16 + quad * 4 + i];
       if (so < 0) continue;
 #pragma unroll
       for (int b = 0; b < 4; b++) {
-        int n = nbase + b * 16 + n16;
+        int n = n0 + wn + b * 16 + n16;
         if (n < N) out[(size_t)so * ldo + n] = __float2bfloat16(acc[a][b][i]);
       }
     }
@@ -263,13 +358,13 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 expert_gemm_fma_k(const T* __restrict__ x, int ldx, int x_div, const T* __restrict__ w,
                   const int* __restrict__ cnt, const int* __restrict__ rows, int ldr,
-                  T* __restrict__ out, int ldo, int N, int K) {
+                  T* __restrict__ out, int ldo, int N, int K, int E, int TMP) {
   __shared__ float sx[32][EG_KT + 1];
   __shared__ float sw[64][EG_KT + 1];
   __shared__ int sslot[32];
-  const int e = blockIdx.z, c = cnt[e];
-  const int m0 = blockIdx.x * 32, n0 = blockIdx.y * 64;
-  if (m0 >= c) return;
+  int e, m0, nt;
+  if (!find_tile(cnt, E, 32, TMP, e, m0, nt)) return;
+  const int c = cnt[e], n0 = nt * 64;
   const int tid = threadIdx.x;
   if (tid < 32) sslot[tid] = m0 + tid < c ? rows[(size_t)e * ldr + m0 + tid] : -1;
   __syncthreads();
@@ -343,28 +438,31 @@ int p2p_sm_group_route(const void* h, int ldh, const float* wr, int R, int W, in
   return (int)hipGetLastError();
 }
 
-// max_slots: the most slots any expert can hold (the grid covers that many)
+// total_slots: slots over all experts (rows * top; every slot is in exactly one list)
 int p2p_sm_expert_gemm(const void* x, int ldx, int x_div, const void* w, const int* cnt,
                        const int* rows, int ldr, void* out, int ldo, int E, int N, int K,
-                       int max_slots, int f32, hipStream_t st) {
-  if (max_slots <= 0 || E <= 0) return 0;
+                       int total_slots, int f32, hipStream_t st) {
+  if (total_slots <= 0 || E <= 0) return 0;
   if (x_div < 1 || N < 1 || K < 1) return (int)hipErrorInvalidValue;
   if (!f32 && K % 8 == 0 && ldx % 8 == 0 && ((size_t)x & 15) == 0 && ((size_t)w & 15) == 0) {
-    if (max_slots >= 512) {   // prompts: the large tile
-      dim3 grid((max_slots + 127) / 128, (N + 127) / 128, E);
+    if (total_slots >= 64 * E) {   // prompts: the large tile
+      int tmp = (((total_slots + 127) / 128 + E) + 7) & ~7;
+      dim3 grid(tmp * ((N + 127) / 128));
       hipLaunchKernelGGL(expert_gemm_mfma_big_k, grid, dim3(256), 0, st, (const bf16*)x, ldx, x_div,
-                         (const bf16*)w, cnt, rows, ldr, (bf16*)out, ldo, N, K);
+                         (const bf16*)w, cnt, rows, ldr, (bf16*)out, ldo, N, K, E, tmp);
       return (int)hipGetLastError();
     }
-    dim3 grid((max_slots + 63) / 64, (N + 63) / 64, E);
+    int tmp = (((total_slots + 15) / 16 + E) + 7) & ~7;
+    dim3 grid(tmp * ((N + 63) / 64));
     hipLaunchKernelGGL(expert_gemm_mfma_k, grid, dim3(256), 0, st, (const bf16*)x, ldx, x_div,
-                       (const bf16*)w, cnt, rows, ldr, (bf16*)out, ldo, N, K);
+                       (const bf16*)w, cnt, rows, ldr, (bf16*)out, ldo, N, K, E, tmp);
     return (int)hipGetLastError();
   }
-  dim3 grid((max_slots + 31) / 32, (N + 63) / 64, E);
+  int tmp = (((total_slots + 31) / 32 + E) + 7) & ~7;
+  dim3 grid(tmp * ((N + 63) / 64));
   SM_DISPATCH_T(f32, hipLaunchKernelGGL(expert_gemm_fma_k<T>, grid, dim3(256), 0, st,
                                          (const T*)x, ldx, x_div, (const T*)w, cnt, rows, ldr,
-                                         (T*)out, ldo, N, K));
+                                         (T*)out, ldo, N, K, E, tmp));
   return (int)hipGetLastError();
 }
 

@@ -105,15 +105,28 @@ def _hybrid_presets() -> dict:
           "mixer": {"heads": 4, "dim": 32, "vdim": 32, "kv_rank": 64, "mask": {"size": 128},
                     "scale": 32 ** -0.5},
           "mlp": {"kind": "dense", "ff": 512, "limit": 7.0}}
+    hg = {"type": "hgrn2", "mixer": {"heads": 4, "dim": 32, "vdim": 64}, "mlp": None}
+    moe = {"kind": "moe", "expert": {"ff": 128, "limit": 7.0},
+           "router": {"experts": 8, "top": 2, "groups": {"count": 4, "keep": 2}}}
+    pa = {"type": "parallel",
+          "mixer": {"left": {"heads": 4, "kv_heads": 2, "dim": 64, "vdim": 64, "mask": {"size": 128},
+                             "rot": {"base": 10000.0, "dims": 32}, "scale": 64 ** -0.5},
+                    "right": {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 64, "conv": 4},
+                    "left_scale": 1.0, "right_scale": 1.0},
+          "mlp": {"kind": "dense", "ff": 512}}
     return {"tiny-regesun": HybridConfig.from_dict(
         {"architecture": "Regesun", "width": 256, "vocab": 512, "max_positions": 4096,
          "norm": {"eps": 1e-5}, "layers": [gd, mb, la, mb, gd, la], "eos_token_id": [2]},
-        name="tiny-regesun")}
+        name="tiny-regesun"),
+        "tiny-rotutar": HybridConfig.from_dict(
+        {"architecture": "Rotutar", "width": 256, "vocab": 512, "norm": {"eps": 1e-5, "groups": 4},
+         "logit_softcap": 30.0, "layers": [hg, dict(hg, mlp=moe), pa, hg, dict(hg, mlp=moe), pa],
+         "eos_token_id": [2]}, name="tiny-rotutar")}
 
 
 def get_config(name: str):
     key = ALIASES.get(name, name)
-    if key not in PRESETS and key.endswith("regesun"):
+    if key not in PRESETS and key.endswith(("regesun", "rotutar")):
         hp = _hybrid_presets()
         if key in hp:
             return hp[key]

@@ -979,10 +979,12 @@ def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows):
     return ids, wts
 
 
-def expert_gemm(x, x_div: int, w, cnt, rows, out, max_slots: int):
+def expert_gemm(x, x_div: int, w, cnt, rows, out, total_slots: int):
     """Per expert e and each of its routed slots s = rows[e, i] (i < cnt[e]):
     out[s] = x[s // x_div] @ w[e]^T.  w [E, N, K] (activation type), x [*, K], out [slots, N].
-    Accumulation is fp32; a slot's result does not depend on the other slots."""
+    total_slots: the slots over all experts (every slot is in exactly one list; the grid is
+    sized from it, so no launch depends on the counts).  Accumulation is fp32; a slot's
+    result does not depend on the other slots."""
     E, N, K = w.shape
     if not x.is_cuda:
         for e in range(E):
@@ -993,10 +995,10 @@ def expert_gemm(x, x_div: int, w, cnt, rows, out, max_slots: int):
     _rows2d(x, "x")
     _rows2d(out, "out")
     assert w.is_contiguous() and x.shape[1] == K and out.shape[1] == N
-    assert x.dtype == w.dtype == out.dtype and rows.stride(0) >= max_slots
+    assert x.dtype == w.dtype == out.dtype and cnt.numel() == E
     _chk(lib().p2p_sm_expert_gemm(x.data_ptr(), x.stride(0), x_div, w.data_ptr(), cnt.data_ptr(),
                                   rows.data_ptr(), rows.stride(0), out.data_ptr(), out.stride(0),
-                                  E, N, K, max_slots, _f32(x), _st(x)), "expert_gemm")
+                                  E, N, K, total_slots, _f32(x), _st(x)), "expert_gemm")
     return out
 
 
