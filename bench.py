@@ -73,6 +73,8 @@ def parse(argv=None):
     ap.add_argument("--hybrid-design", choices=("regesun", "rotutar", "both"), default="regesun",
                     help="regesun: Regesun beside the Llama; rotutar: Rotutar beside Regesun "
                          "(equal width and depth); both: all three")
+    ap.add_argument("--hybrid-phase", choices=("both", "prefill", "decode"), default="both",
+                    help="measure only the prompt or only the decode workload (profiling)")
     ap.add_argument("--hybrid-only", default=None,
                     help="run only the models whose name contains this (profiling one model)")
     ap.add_argument("--hybrid-sizes", default="1024,2048", help="model widths for --hybrid")

@@ -87,12 +87,14 @@ def llama_like(width: int, layers: int, params: int):
                        rope_llama3=None, bos_id=1, eos_ids=(2,))
 
 
-def measure(eng, vocab, prompt, batch, ctx, new_tokens, steps, warmup, dev):
+def measure(eng, vocab, prompt, batch, ctx, new_tokens, steps, warmup, dev, phase="both"):
     g = torch.Generator().manual_seed(0)
     long_p = [torch.randint(3, vocab, (prompt,), generator=g).tolist()]
     many = [torch.randint(3, vocab, (ctx,), generator=g).tolist() for _ in range(batch)]
     out = {}
     for name, prompts, new in (("prefill", long_p, 2), ("decode", many, new_tokens)):
+        if phase not in ("both", name):
+            continue
         for _ in range(warmup):
             eng.generate(prompts, new, stop_on_eos=False)
         torch.cuda.synchronize(dev)
@@ -139,7 +141,8 @@ def run(a):
                              max_batch=batch)
                 eng.warmup((batch,), ctx=ctx + new)
             t0 = time.perf_counter()
-            m = measure(eng, cfg.vocab, prompt, batch, ctx, new, a.steps, a.warmup, dev)
+            m = measure(eng, cfg.vocab, prompt, batch, ctx, new, a.steps, a.warmup, dev,
+                        getattr(a, "hybrid_phase", "both"))
             line = {"metric": "hybrid-vs-dense throughput", "model": cfg.name,
                     "params_m": round((params if hybrid else cfg.n_params()) / 1e6, 1),
                     "width": width, "layers": cfg.n_layers, "dtype": "bf16",

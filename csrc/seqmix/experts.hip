@@ -1,10 +1,10 @@
 // Mixture of experts: the router with a group-limited choice, the expert matrix products over
 // the routed rows, and the weighted sum of the chosen experts' outputs.
 //
-// group_route_k: z = h . Wr^T in fp32, s = sigmoid(z).  The E experts form `groups` equal groups
-// of neighbours; a group's score is the sum of its two largest s; only experts of the best
-// `keep` groups can be chosen, and among them the `top` largest s win (ties: the lower index).
-// The weights are the chosen s as they are.  A token r routed to its k-th expert is slot
+// group_route_k: z = h . Wr^T in fp32, s = sigmoid(z).  The E experts are cut into `groups`
+// contiguous blocks of equal size; a block is ranked by its top-2 sum of s; experts outside the
+// `keep` best blocks are struck out, and the `top` largest remaining s win (ties: the lower
+// index).  The weights are the winners' s without rescaling.  A token r routed to its k-th expert is slot
 // r * top + k; every expert gets the list of its slots (cnt / rows).
 //
 // expert_gemm: for expert e and each of its slots s: out[s] = x[s / x_div] . W_e^T.  Rows are
@@ -80,7 +80,7 @@ group_route_k(const T* __restrict__ h, int ldh, const float* __restrict__ wr, in
   const int per = E / groups;
   if (keep < groups) {
     for (int g = lane; g < groups; g += 64) {
-      float b1 = -1.0f, b2 = -1.0f;   // the two largest of the group
+      float b1 = -1.0f, b2 = -1.0f;   // top-2 of the block
       for (int i = 0; i < per; i++) {
         float v = ss[g * per + i];
         if (v > b1) { b2 = b1; b1 = v; }

@@ -3,13 +3,14 @@
 //   S <- diag(g) S
 //   u = v                        plain write   (HGRN2: g = f, k = 1 - f)
 //   u = beta * (v - S^T k)       delta rule    (the write corrects what the key reads)
-//   S <- S + k u^T,  o = S^T q   (the read-out sees the token's own write)
+//   S <- S + k u^T,  o = S^T q   (o is formed from the updated S)
 // followed by the head's RMS norm over V, a weight shared by the heads and, for the delta
 // rule, a sigmoid output gate.
 //
 // The value columns of S are independent.  A wavefront covers 16 columns x 4 slices of the key
-// index; lane (c, s) keeps rows s*DQ .. s*DQ+DQ-1 of column c in registers, and the sums over
-// the key index (S^T k before the write, S^T q after it) are finished with two lane shuffles.
+// index; lane (c, s) keeps rows s*DQ .. s*DQ+DQ-1 of column c in registers (NC columns, 16
+// apart, in the general form of the kernel), and the sums over the key index (S^T k before
+// the write, S^T q after it) are finished with two lane shuffles.
 // The tokens of a sequence portion are walked in order; their vectors are staged through LDS
 // a chunk at a time and everything that enters the recurrence is evaluated in fp32 while
 // staging: HGRN2's silu(q) and f = lower + (1 - lower) sigmoid(. + b); the delta rule's unit q
@@ -51,16 +52,17 @@ struct ScanArgs {
   float* chunk_trans;   // [chunks, H, D, D]
 };
 
-template <typename T, int DQ, bool DELTA>
-__global__ void __launch_bounds__(1024) gated_scan_k(ScanArgs a) {
+template <typename T, int DQ, bool DELTA, int NC>
+__global__ void __launch_bounds__(1024 / NC) gated_scan_k(ScanArgs a) {
   constexpr int DKP = 4 * DQ;   // padded key index (zero filled in LDS)
+  constexpr int WC = 16 * NC;   // columns per wavefront: a lane keeps NC columns, 16 apart
   const int H = a.H, D = a.D, V = a.V, CT = a.CT, mode = a.mode;
   const int e = blockIdx.x / H, h = blockIdx.x % H;
   const Entry en = load_entry(a.ent, e);
   if (en.n <= 0) return;
   const bool trans = mode == 3;
-  const int NC = trans ? D : V;                // columns of the matrix this block carries
-  const int nw = blockDim.x >> 6, VP = nw * 16;
+  const int NCOL = trans ? D : V;              // columns of the matrix this block carries
+  const int nw = blockDim.x >> 6, VP = nw * WC;
   extern __shared__ __align__(16) float smem[];
   float* sq = smem;                  // [CT][DKP]
   float* sk = sq + CT * DKP;
@@ -70,27 +72,35 @@ __global__ void __launch_bounds__(1024) gated_scan_k(ScanArgs a) {
   float* sb = so + CT * VP;          // [CT]
   float* sP = sb + CT;               // [DKP] product of the chunk's decays (mode 1, plain write)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int j = wave * 16 + (lane & 15), is = lane >> 4, i0 = is * DQ;
-  const bool act = j < NC;
-  const int jc = min(j, NC - 1);
+  const int is = lane >> 4, i0 = is * DQ;
+  int j[NC], jc[NC];
+  bool act[NC];
+#pragma unroll
+  for (int c = 0; c < NC; c++) {
+    j[c] = wave * WC + c * 16 + (lane & 15);
+    act[c] = j[c] < NCOL;
+    jc[c] = min(j[c], NCOL - 1);
+  }
   const int hk = DELTA ? h / (H / a.G) : h;    // the q/k head this head reads
   const T* proj = (const T*)a.proj;
   const T* araw = (const T*)a.araw;
   const T* braw = (const T*)a.braw;
   const T* gate = (const T*)a.gate;
   T* out = (T*)a.out;
-  float S[DQ];
+  float S[NC][DQ];
   float* Sg = mode == 0 ? a.state + ((size_t)en.slot * H + h) * D * V
             : trans     ? a.chunk_trans + ((size_t)en.slot * H + h) * D * D
                         : a.chunk_state + ((size_t)en.slot * H + h) * D * V;
   const bool from_state = mode == 2 || (mode == 0 && en.start > 0);
 #pragma unroll
-  for (int q = 0; q < DQ; q++) {
-    // loads at clamped addresses, selected afterwards, so that they go out together
-    float v0 = (trans && i0 + q == j) ? 1.0f : 0.0f;
-    float vv = from_state ? Sg[(size_t)min(i0 + q, D - 1) * NC + jc] : v0;
-    S[q] = (act && i0 + q < D) ? vv : 0.0f;
-  }
+  for (int c = 0; c < NC; c++)
+#pragma unroll
+    for (int q = 0; q < DQ; q++) {
+      // loads at clamped addresses, selected afterwards, so that they go out together
+      float v0 = (trans && i0 + q == j[c]) ? 1.0f : 0.0f;
+      float vv = from_state ? Sg[(size_t)min(i0 + q, D - 1) * NCOL + jc[c]] : v0;
+      S[c][q] = (act[c] && i0 + q < D) ? vv : 0.0f;
+    }
   if (!DELTA && mode == 1)
     for (int i = threadIdx.x; i < DKP; i += blockDim.x) sP[i] = 1.0f;
   const float negA = DELTA ? -expf(a.A_log[h]) : 0.0f;
@@ -158,40 +168,62 @@ __global__ void __launch_bounds__(1024) gated_scan_k(ScanArgs a) {
       const float4* k4 = (const float4*)(sk + t * DKP + i0);
       const float4* g4 = (const float4*)(sg + t * DKP + i0);
       const float4* q4 = (const float4*)(sq + t * DKP + i0);
-      float u = trans ? 0.0f : sv[t * VP + jc];
+      float u[NC];
+#pragma unroll
+      for (int c = 0; c < NC; c++) u[c] = trans ? 0.0f : sv[t * VP + jc[c]];
       if (DELTA) {
-        float d0 = 0.0f, d1 = 0.0f, d2 = 0.0f, d3 = 0.0f;   // four chains instead of one
+        float d0[NC], d1[NC];   // two chains per column instead of one
+#pragma unroll
+        for (int c = 0; c < NC; c++) d0[c] = d1[c] = 0.0f;
 #pragma unroll
         for (int q = 0; q < DQ / 4; q++) {
           float4 g = g4[q], k = k4[q];
-          S[4 * q] *= g.x; S[4 * q + 1] *= g.y; S[4 * q + 2] *= g.z; S[4 * q + 3] *= g.w;
-          d0 += k.x * S[4 * q]; d1 += k.y * S[4 * q + 1];
-          d2 += k.z * S[4 * q + 2]; d3 += k.w * S[4 * q + 3];
+#pragma unroll
+          for (int c = 0; c < NC; c++) {
+            S[c][4 * q] *= g.x; S[c][4 * q + 1] *= g.y; S[c][4 * q + 2] *= g.z; S[c][4 * q + 3] *= g.w;
+            d0[c] += k.x * S[c][4 * q] + k.z * S[c][4 * q + 2];
+            d1[c] += k.y * S[c][4 * q + 1] + k.w * S[c][4 * q + 3];
+          }
         }
-        float d = (d0 + d1) + (d2 + d3);
-        d += __shfl_xor(d, 16, 64);
-        d += __shfl_xor(d, 32, 64);
-        u = sb[t] * (u - d);
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+          float d = d0[c] + d1[c];
+          d += __shfl_xor(d, 16, 64);
+          d += __shfl_xor(d, 32, 64);
+          u[c] = sb[t] * (u[c] - d);
+        }
       } else {
 #pragma unroll
         for (int q = 0; q < DQ / 4; q++) {
           float4 g = g4[q];
-          S[4 * q] *= g.x; S[4 * q + 1] *= g.y; S[4 * q + 2] *= g.z; S[4 * q + 3] *= g.w;
+#pragma unroll
+          for (int c = 0; c < NC; c++) {
+            S[c][4 * q] *= g.x; S[c][4 * q + 1] *= g.y; S[c][4 * q + 2] *= g.z; S[c][4 * q + 3] *= g.w;
+          }
         }
       }
-      float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
+      float o0[NC], o1[NC];
+#pragma unroll
+      for (int c = 0; c < NC; c++) o0[c] = o1[c] = 0.0f;
 #pragma unroll
       for (int q = 0; q < DQ / 4; q++) {
         float4 k = k4[q], qv = q4[q];
-        S[4 * q] += k.x * u; S[4 * q + 1] += k.y * u; S[4 * q + 2] += k.z * u; S[4 * q + 3] += k.w * u;
-        o0 += S[4 * q] * qv.x; o1 += S[4 * q + 1] * qv.y;
-        o2 += S[4 * q + 2] * qv.z; o3 += S[4 * q + 3] * qv.w;
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+          S[c][4 * q] += k.x * u[c]; S[c][4 * q + 1] += k.y * u[c];
+          S[c][4 * q + 2] += k.z * u[c]; S[c][4 * q + 3] += k.w * u[c];
+          o0[c] += S[c][4 * q] * qv.x + S[c][4 * q + 2] * qv.z;
+          o1[c] += S[c][4 * q + 1] * qv.y + S[c][4 * q + 3] * qv.w;
+        }
       }
       if (mode == 0 || mode == 2) {
-        float o = (o0 + o1) + (o2 + o3);
-        o += __shfl_xor(o, 16, 64);
-        o += __shfl_xor(o, 32, 64);
-        if (is == 0) so[t * VP + j] = act ? o : 0.0f;
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+          float o = o0[c] + o1[c];
+          o += __shfl_xor(o, 16, 64);
+          o += __shfl_xor(o, 32, 64);
+          if (is == 0) so[t * VP + j[c]] = act[c] ? o : 0.0f;
+        }
       }
     }
     __syncthreads();
@@ -212,10 +244,14 @@ __global__ void __launch_bounds__(1024) gated_scan_k(ScanArgs a) {
     // written again only after the next staging barrier, which every wave reaches after its
     // share of this chunk's outputs
   }
-  if (act && mode != 2) {
+  if (mode != 2) {
 #pragma unroll
-    for (int q = 0; q < DQ; q++)
-      if (i0 + q < D) Sg[(size_t)(i0 + q) * NC + j] = S[q];
+    for (int c = 0; c < NC; c++)
+      if (act[c]) {
+#pragma unroll
+        for (int q = 0; q < DQ; q++)
+          if (i0 + q < D) Sg[(size_t)(i0 + q) * NCOL + j[c]] = S[c][q];
+      }
   }
   if (!DELTA && mode == 1) {
     __syncthreads();
@@ -246,21 +282,25 @@ diag_chain_k(float* __restrict__ cs, const float* __restrict__ decay, float* __r
 }
 
 // Chain of the delta rule: init_{c+1} = T_c . init_c + local_c with a dense D x D transition.
-// The columns of the state are independent: one block per (portion, head, 16 columns), the
-// current columns in LDS, thread (column, row group) forms every 16th row of the product.
-#define DC_ROWS 16   // rows per thread at most (D <= 256)
+// The columns of the state are independent: one block per (portion, head, 8 columns), the
+// current columns in LDS, thread (column, row group) forms every 32nd row of the product.
+#define DC_COLS 8
+#define DC_RG 32     // row groups: 256 threads / DC_COLS
+#define DC_ROWS 8    // rows per thread at most (D <= 256)
 __global__ void __launch_bounds__(256)
 dense_chain_k(float* __restrict__ cs, const float* __restrict__ trans, float* __restrict__ state,
               const int* __restrict__ cent, int H, int D, int V) {
-  extern __shared__ float scur[];   // [D][17]
+  extern __shared__ float scur[];   // [D][DC_COLS + 1]
+  constexpr int LD = DC_COLS + 1;
   const int e = blockIdx.y / H, h = blockIdx.y % H;
-  const int col = threadIdx.x & 15, rg = threadIdx.x >> 4;
-  const int j = blockIdx.x * 16 + col;
+  const int col = threadIdx.x % DC_COLS, rg = threadIdx.x / DC_COLS;
+  const int j = blockIdx.x * DC_COLS + col;
   const bool act = j < V;
   const int jc = min(j, V - 1);
   const int c0 = cent[4 * e], nc = cent[4 * e + 1], start = cent[4 * e + 2], slot = cent[4 * e + 3];
   float* sg = state + ((size_t)slot * H + h) * D * V;
-  for (int i = rg; i < D; i += 16) scur[i * 17 + col] = (start > 0 && act) ? sg[(size_t)i * V + jc] : 0.0f;
+  for (int i = rg; i < D; i += DC_RG)
+    scur[i * LD + col] = (start > 0 && act) ? sg[(size_t)i * V + jc] : 0.0f;
   __syncthreads();
   for (int c = c0; c < c0 + nc; c++) {
     float* loc = cs + ((size_t)c * H + h) * D * V;
@@ -268,32 +308,32 @@ dense_chain_k(float* __restrict__ cs, const float* __restrict__ trans, float* __
     float nv[DC_ROWS];
 #pragma unroll
     for (int r = 0; r < DC_ROWS; r++) {
-      int i = rg + 16 * r;
+      int i = rg + DC_RG * r;
       if (i < D) {
         float acc0 = loc[(size_t)i * V + jc], acc1 = 0.0f;
         const float* Ti = Tc + (size_t)i * D;
         int k = 0;
         for (; k + 3 < D; k += 4) {
-          acc0 += Ti[k] * scur[k * 17 + col] + Ti[k + 2] * scur[(k + 2) * 17 + col];
-          acc1 += Ti[k + 1] * scur[(k + 1) * 17 + col] + Ti[k + 3] * scur[(k + 3) * 17 + col];
+          acc0 += Ti[k] * scur[k * LD + col] + Ti[k + 2] * scur[(k + 2) * LD + col];
+          acc1 += Ti[k + 1] * scur[(k + 1) * LD + col] + Ti[k + 3] * scur[(k + 3) * LD + col];
         }
-        for (; k < D; k++) acc0 += Ti[k] * scur[k * 17 + col];
+        for (; k < D; k++) acc0 += Ti[k] * scur[k * LD + col];
         nv[r] = acc0 + acc1;
       }
     }
     __syncthreads();   // every thread has read the old columns
 #pragma unroll
     for (int r = 0; r < DC_ROWS; r++) {
-      int i = rg + 16 * r;
+      int i = rg + DC_RG * r;
       if (i < D) {
-        if (act) loc[(size_t)i * V + j] = scur[i * 17 + col];   // init_c replaces local_c
-        scur[i * 17 + col] = nv[r];
+        if (act) loc[(size_t)i * V + j] = scur[i * LD + col];   // init_c replaces local_c
+        scur[i * LD + col] = nv[r];
       }
     }
     __syncthreads();
   }
   if (act)
-    for (int i = rg; i < D; i += 16) sg[(size_t)i * V + j] = scur[i * 17 + col];
+    for (int i = rg; i < D; i += DC_RG) sg[(size_t)i * V + j] = scur[i * LD + col];
 }
 
 template <bool DELTA>
@@ -302,20 +342,23 @@ static int launch_scan(ScanArgs a, int E, int f32, hipStream_t st) {
   if (a.H < 1 || a.D < 1 || a.V < 1 || a.D > 256 || a.V > 256 || a.G < 1 || a.H % a.G)
     return (int)hipErrorInvalidValue;
   int cols = a.mode == 3 ? a.D : a.V;
-  int nw = (cols + 15) / 16;
   int dq = a.D <= 32 ? 8 : a.D <= 64 ? 16 : a.D <= 128 ? 32 : 64;
-  int per_tok = 3 * 4 * dq + 2 * nw * 16 + 1;
+  // one column per lane: two (NC = 2) halve the wavefronts that read the staged vectors from
+  // LDS but measured no faster (120 us against 110 us per 64-token pass at 128 x 128 states)
+  const int nc = 1;
+  int nw = (cols + 16 * nc - 1) / (16 * nc);
+  int per_tok = 3 * 4 * dq + 2 * nw * 16 * nc + 1;
   int CT = 16;
   while (CT > 2 && (size_t)(CT * per_tok + 4 * dq) * 4 > 48 * 1024) CT /= 2;
   a.CT = CT;
   size_t shm = (size_t)(CT * per_tok + 4 * dq) * 4;
   dim3 grid(E * a.H), block(64 * nw);
-#define GS(DQ)                                                                              \
-  SM_DISPATCH_T(f32, hipLaunchKernelGGL((gated_scan_k<T, DQ, DELTA>), grid, block, shm, st, a))
-  if (dq == 8) GS(8);
-  else if (dq == 16) GS(16);
-  else if (dq == 32) GS(32);
-  else GS(64);
+#define GS(DQ, NC)                                                                            \
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL((gated_scan_k<T, DQ, DELTA, NC>), grid, block, shm, st, a))
+  if (dq == 8) GS(8, 1);
+  else if (dq == 16) GS(16, 1);
+  else if (dq == 32) GS(32, 1);
+  else GS(64, 1);
 #undef GS
   return (int)hipGetLastError();
 }
@@ -335,8 +378,8 @@ static int launch_chunked(ScanArgs a, const int* vent, int NV, const int* cent, 
   if (DELTA) {
     a.mode = 3;
     if ((err = launch_scan<DELTA>(a, NV, f32, st))) return err;
-    hipLaunchKernelGGL(dense_chain_k, dim3((a.V + 15) / 16, E * a.H), dim3(256),
-                       (size_t)a.D * 17 * 4, st, cs, ct, state, cent, a.H, a.D, a.V);
+    hipLaunchKernelGGL(dense_chain_k, dim3((a.V + DC_COLS - 1) / DC_COLS, E * a.H), dim3(256),
+                       (size_t)a.D * (DC_COLS + 1) * 4, st, cs, ct, state, cent, a.H, a.D, a.V);
   } else {
     hipLaunchKernelGGL(diag_chain_k, dim3((a.D * a.V + 255) / 256, E * a.H), dim3(256), 0, st, cs,
                        cd, state, cent, a.H, a.D, a.V);

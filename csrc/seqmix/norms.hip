@@ -218,7 +218,10 @@ int p2p_sm_gate_norm_add(float* x, const void* y, int ldy, const void* g, int ld
                          void* h, int ldh, int h_f32, int f32, hipStream_t st) {
   if (R <= 0) return 0;
   if (parts <= 0 || n % parts || (h && h_f32 != f32)) return (int)hipErrorInvalidValue;
-  SM_DISPATCH_T(f32, hipLaunchKernelGGL(gate_norm_add_k<T>, dim3(R * parts), dim3(256), 0, st, x,
+  // many short parts (prompts): one wavefront per (row, part), so the reduction needs no other
+  // wave and more parts are in flight; few rows (decode) keep four wavefronts per part
+  const int threads = (n / parts <= 1024 && R * parts >= 1024) ? 64 : 256;
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(gate_norm_add_k<T>, dim3(R * parts), dim3(threads), 0, st, x,
                                          (const T*)y, ldy, (const T*)g, ldg, gb, w, n, parts, eps,
                                          (T*)h, ldh));
   return (int)hipGetLastError();

@@ -3,15 +3,16 @@
 // not take).
 //
 // qk_norm_rope_store_k: one projection buffer holds q (H heads x D) | k (G x D) | v (G x V) of a
-// row.  q and k are RMS-normalised over their whole rows (all heads at once), weighted, and the
-// channel pairs (2i, 2i+1), i < nrot, of every head are turned by the angle pos * inv_freq[i]:
+// row.  q and k are RMS-normalised with one mean square per row (heads not separated) and
+// weighted, and the channel pairs (2i, 2i+1), i < nrot, of every head are turned by the angle
+// pos * inv_freq[i]:
 // (a, b) -> (a cos - b sin, b cos + a sin).  q goes to its own buffer, k | v to the row of the
 // paged pool that the token owns.  Norm, angle and rotation are fp32.
 //
 // window_attn_k: pool row = [k of G heads | v of G heads]; query head h reads key/value head
 // h / (H/G).  Causal sliding window: position i sees j with 0 <= i - j < win.  The softmax
-// denominator holds one more term exp(sink_h) with no key and no value: the running maximum
-// starts at sink_h and the running sum at 1.  One block per (query row, key/value head): the
+// denominator holds one more term exp(sink_h) that adds nothing to the numerator: the running
+// maximum starts at sink_h and the running sum at 1.  One block per (query row, key/value head): the
 // heads of the group share the key and value tiles, which stream through LDS with an online
 // softmax.
 #include "common.h"

@@ -5,8 +5,9 @@ optionally a feed-forward (``FEEDFORWARDS``).  A design (``DESIGNS``) fixes how 
 is wrapped around the residual stream,
 
     "sandwich"    x <- x + scale * norm_b(f(norm_a(x)))      RMS norms, per-channel layer scale
-    "gated_post"  x <- x + norm(f(x) * sigmoid(R x + b))     the sublayer reads x itself; the
-                                                             norm is taken in equal parts
+    "gated_post"  x <- x + norm(f(x) * sigmoid(R x + b))     no norm on the way in; the norm
+                                                             on the way out is taken in
+                                                             equal parts of the vector
 
 and whether learned absolute positions are added to the token embedding.  Mixers:
 
@@ -17,11 +18,11 @@ and whether learned absolute positions are added to the token embedding.  Mixers
                         are up-projections of it), causal sliding window, softmax with a
                         learned per-head sink, sigmoid output gate, no positional rotation;
   ``window_attention``  grouped-query attention over cached keys and values: RMS norm of the
-                        whole query / key projection, interleaved rotary positions on the
+                        whole query / key projection, rotary positions on adjacent channel pairs of the
                         first channels of each head, causal sliding window, softmax sink;
   ``gated_delta``       gated delta rule: short causal convolutions + silu on q, k, v, unit
                         keys, a per-channel decay and a write that corrects what the key reads;
-  ``hgrn2``             linear attention whose forget gate also sets what is written;
+  ``hgrn2``             gated linear attention: the write strength is 1 - forget gate;
   ``parallel``          two mixers side by side on the same input, summed with fixed scales.
 
 Feed-forwards: ``dense`` (silu-gated, or the clamped gated unit when the config gives a
@@ -617,7 +618,7 @@ class DenseFF:
 class MoEFF:
     """Mixture of clamped gated experts behind a sigmoid router whose choice is limited to
     the best groups of experts (``ops.seqmix.group_route``); the chosen experts' scores weight
-    their outputs as they are.  The expert products run grouped over the routed rows
+    their outputs without rescaling.  The expert products run grouped over the routed rows
     (``ops.seqmix.expert_gemm``)."""
     w_in = None   # the router and the grouped products read the input themselves
 
@@ -837,7 +838,7 @@ class HybridModel:
 
     def _forward_gated_post(self, b: StepBatch, layer_out=None):
         """x <- x + N(f(x) * sigmoid(R x + b)) per sublayer: the sublayer and its gate read the
-        residual rows as they are (rounded to the activation type), so one matrix product
+        un-normalised residual rows (rounded to the activation type), so one matrix product
         serves both; the pass that adds the result also writes the next sublayer's input."""
         cfg, w = self.cfg, self.w
         x = torch.empty(b.R, cfg.width, device=self.device, dtype=torch.float32)

@@ -625,7 +625,7 @@ def gate_norm_add(x, y, g, gb, w, parts: int, eps: float, next_out=None):
     """x += N(y * sigmoid(g + gb)) * w on the fp32 residual x, N the RMS norm taken separately
     over ``parts`` equal parts of the row.  y, g: activation-typed [R, n] (g the gate's
     projection before its bias gb).  next_out (activation type): the updated rows, which the
-    next sublayer reads as they are."""
+    next sublayer takes as its input without a norm of its own."""
     R, n = x.shape
     if not x.is_cuda:
         v = y.float() * torch.sigmoid(g.float() + gb)
@@ -691,7 +691,7 @@ def rope_inv_freq(base: float, dims: int, device) -> torch.Tensor:
 def qk_norm_rope_store(proj, H: int, G: int, D: int, V: int, qw, kw, inv_freq, pos, cache_rows,
                        pool, eps: float, q_out):
     """Prepares attention inputs from one projection buffer proj = [q (H*D) | k (G*D) | v (G*V)]:
-    q and k are RMS-normalised over their whole rows (all heads at once) with weights qw / kw,
+    q and k are RMS-normalised with one mean square per row (heads not separated) and weights qw / kw,
     then channels (2i, 2i+1), i < len(inv_freq), of every head are rotated by pos * inv_freq[i].
     q goes to q_out [R, H*D]; k | v go to the paged pool rows ``cache_rows`` ([tokens,
     G*D + G*V]).  Norm, angles and the rotation are fp32."""
@@ -821,7 +821,7 @@ def window_attn(q, pool, block_tables, row_ent, pos, sink, scale: float, win: in
 # Per head a D x V fp32 state S (key channel i, value channel j), one step per token:
 #   S <- diag(g) S;   u = v                      (plain write)
 #                     u = beta * (v - S^T k)     (delta rule: the write corrects what k reads)
-#   S <- S + k u^T;   o = S^T q                  (the read-out sees the token's own write)
+#   S <- S + k u^T;   o = S^T q                  (o is formed from the updated S)
 # HGRN2 is the plain write with g = f and k = 1 - f; the gated delta rule has its own key.
 def hgrn2_scan(proj, lower, fb, normw, state, ent, ent_host, out, H: int, D: int, V: int,
                eps: float, out_scale: float = 1.0):
@@ -940,8 +940,9 @@ def gated_delta_scan(conv, araw, braw, gate, A_log, dt_bias, normw, state, ent, 
 # ------------------------------------------------------------------ mixture of experts
 def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows):
     """Sigmoid router with group-limited choice.  z = h wr^T in fp32 (wr fp32 [E, W]),
-    s = sigmoid(z); the E experts form ``groups`` equal groups of neighbours, a group scores the
-    sum of its two largest s, only experts of the best ``keep`` groups can be chosen; the
+    s = sigmoid(z); the E experts are cut into ``groups`` contiguous blocks of equal size, a
+    block is ranked by its top-2 sum of s, experts outside the ``keep`` best blocks are
+    struck out; the
     ``top`` largest s among them win (ties: the lower index), their weights are their s.
     ids int32 / wts fp32 [R, top]; cnt int32 [E] and rows int32 [E, R*top] list per expert the
     slots (row * top + k) routed to it (cnt is cleared here)."""

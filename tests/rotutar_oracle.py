@@ -67,7 +67,7 @@ def window_attention(h, t, p, mx, eps):
 
 # ------------------------------------------------------------------ gated delta rule
 def short_conv(x, w):
-    """x [T, C], w [C, taps]: y[t] = sum_j w[:, taps-1-j] * x[t-j], zeros before the start."""
+    """x [T, C], w [C, taps]: y[t] = sum_j w[:, taps-1-j] * x[t-j], with x[t] = 0 for t < 0."""
     T, C = x.shape
     K = w.shape[1]
     y = torch.zeros_like(x)

@@ -126,7 +126,7 @@ def test_layers_match_oracle(dev):
 
 def test_oracle_pieces():
     """The oracle's own building blocks on cases that can be worked out by hand."""
-    # routing: 2 groups of 3; group scores are sums of the two largest sigmoids
+    # routing: 2 blocks of 3 experts, ranked by their top-2 sums of sigmoids
     z = torch.tensor([4.0, -9.0, -9.0, 2.0, 2.1, -9.0], dtype=torch.float64)
     ch, w = O.route(z, {"experts": 6, "top": 2, "groups": {"count": 2, "keep": 1}})
     assert ch == [4, 3]                      # expert 0 is the largest but its group loses
