@@ -56,7 +56,7 @@ def rotutar_config(width: int):
           "mlp": {"kind": "dense", "ff": 4 * width}}
     return HybridConfig.from_dict(
         {"architecture": "Rotutar", "width": width, "vocab": 32000,
-         "norm": {"eps": 1e-5, "groups": 4}, "logit_softcap": 30.0,
+         "norm": {"eps": 1e-5, "groups": 4}, "logit_softcap": 50.0,
          "layers": [hg, dict(hg, mlp=moe), hg, pa] * 4}, name="rotutar-w%d" % width)
 
 

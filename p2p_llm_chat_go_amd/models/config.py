@@ -120,7 +120,7 @@ def _hybrid_presets() -> dict:
         name="tiny-regesun"),
         "tiny-rotutar": HybridConfig.from_dict(
         {"architecture": "Rotutar", "width": 256, "vocab": 512, "norm": {"eps": 1e-5, "groups": 4},
-         "logit_softcap": 30.0, "layers": [hg, dict(hg, mlp=moe), pa, hg, dict(hg, mlp=moe), pa],
+         "logit_softcap": 50.0, "layers": [hg, dict(hg, mlp=moe), pa, hg, dict(hg, mlp=moe), pa],
          "eos_token_id": [2]}, name="tiny-rotutar")}
 
 

@@ -73,8 +73,9 @@ ATTN_SHAPES = [
     (6, 2, 24, 40, 16, 37),      # three heads per key/value head, part of the head rotated
     (4, 4, 16, 8, 16, 1000),     # one head per key/value head, window never reached
     (5, 1, 40, 72, 0, 1),        # no rotation, window of one
-    (16, 2, 96, 96, 96, 100),    # eight heads per key/value head
+    (16, 2, 80, 112, 80, 100),   # eight heads per key/value head
     (34, 2, 8, 16, 4, 70),       # more heads per key/value head than a wavefront's pairs
+    (3, 1, 7, 5, 4, 11),         # odd sizes: the last channel of a head has no partner
 ]
 
 
@@ -112,14 +113,16 @@ def test_window_attention(dt, H, G, D, V, rot, win):
             o2 = torch.empty(R, H * V + 8, dtype=dt, device=DEV)[:, 8:]
             units = None
             if mfma:
-                assert sm.window_mfma_ok(q2, pool2, D, V)
+                if not sm.window_mfma_ok(q2, pool2, D, V):
+                    assert D % 8 or V % 8    # only sizes off the 16-byte grid stay off the matrix cores
+                    continue
                 units = sm.make_units(ent, sm.window_rows_per_wave(H // G)).to(DEV)
             sm.window_attn(q2, pool2, *_d(bt, row_ent, pos, sink), 0.3, win, o2, PAGE, H, G, D, V,
                            units=units, max_keys=max_keys, out_scale=0.7)
             torch.testing.assert_close(o2.cpu().float(), o1.float(), **_tol(dt))
 
 
-SCAN_SHAPES = [(3, 3, 20, 12), (4, 2, 64, 32), (2, 1, 40, 72), (1, 1, 130, 200), (6, 6, 8, 16)]
+SCAN_SHAPES = [(3, 3, 20, 12), (4, 2, 56, 24), (2, 1, 40, 72), (1, 1, 130, 200), (6, 6, 8, 16)]
 
 
 # portions walked token by token / long portions cut into chunks that run side by side
