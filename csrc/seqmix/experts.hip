@@ -177,6 +177,17 @@ __device__ __forceinline__ bool find_tile(const int* __restrict__ cnt, int E, in
   return e >= 0;
 }
 
+// Epilogue with the experts' activation (epi = 1): the weight rows of the first product are
+// stored as 16 gate rows, their 16 up rows, the next 16 gate rows, ..., so a thread that holds
+// output column c of a 16-column tile holds the matching up value in the next tile, and
+//   y = min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, -limit, limit) + 1)
+// is written to column (tile / 2) * 16 + c of an output half as wide.
+__device__ __forceinline__ float expert_act(float g, float u, float limit, float alpha) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g * sigmoidf_(alpha * g) * (u + 1.0f);
+}
+
 // bf16 on the matrix cores, few slots per expert (decode-sized steps): a block takes 16 slots x
 // 64 output columns of one expert and its four wavefronts split K among themselves, so the
 // chain of dependent loads is a quarter as long; each wavefront walks its share in steps of 32
@@ -186,7 +197,7 @@ __device__ __forceinline__ bool find_tile(const int* __restrict__ cnt, int E, in
 __global__ void __launch_bounds__(256)
 expert_gemm_mfma_k(const bf16* __restrict__ x, int ldx, int x_div, const bf16* __restrict__ w,
                    const int* __restrict__ cnt, const int* __restrict__ rows, int ldr,
-                   bf16* __restrict__ out, int ldo, int N, int K, int E, int TMP) {
+                   bf16* __restrict__ out, int ldo, int N, int K, int E, int TMP, int epi, float limit, float alpha) {
   __shared__ f32x4 red[3][4][64];
   int e, m0, nt;
   if (!find_tile(cnt, E, 16, TMP, e, m0, nt)) return;
@@ -245,6 +256,16 @@ expert_gemm_mfma_k(const bf16* __restrict__ x, int ldx, int x_div, const bf16* _
   for (int i = 0; i < 4; i++) {
     int so = __shfl(slot, quad * 4 + i, 64);
     if (so < 0) continue;
+    if (epi) {
+#pragma unroll
+      for (int t = 0; t < 4; t += 2) {
+        int n = n0 + t * 16;
+        if (n + 16 + n16 < N)
+          out[(size_t)so * ldo + n / 2 + n16] =
+              __float2bfloat16(expert_act(acc[t][i], acc[t + 1][i], limit, alpha));
+      }
+      continue;
+    }
 #pragma unroll
     for (int t = 0; t < 4; t++) {
       int n = n0 + t * 16 + n16;
@@ -262,7 +283,7 @@ expert_gemm_mfma_k(const bf16* __restrict__ x, int ldx, int x_div, const bf16* _
 __global__ void __launch_bounds__(256)
 expert_gemm_mfma_big_k(const bf16* __restrict__ x, int ldx, int x_div, const bf16* __restrict__ w,
                        const int* __restrict__ cnt, const int* __restrict__ rows, int ldr,
-                       bf16* __restrict__ out, int ldo, int N, int K, int E, int TMP) {
+                       bf16* __restrict__ out, int ldo, int N, int K, int E, int TMP, int epi, float limit, float alpha) {
   __shared__ __align__(16) unsigned short sA[128 * EB_LD];
   __shared__ __align__(16) unsigned short sB[128 * EB_LD];
   __shared__ int sslot[128];
@@ -343,6 +364,16 @@ expert_gemm_mfma_big_k(const bf16* __restrict__ x, int ldx, int x_div, const bf1
     for (int i = 0; i < 4; i++) {
       int so = sslot[wm + a * 16 + quad * 4 + i];
       if (so < 0) continue;
+      if (epi) {
+#pragma unroll
+        for (int b = 0; b < 4; b += 2) {
+          int n = n0 + wn + b * 16;
+          if (n + 16 + n16 < N)
+            out[(size_t)so * ldo + n / 2 + n16] =
+                __float2bfloat16(expert_act(acc[a][b][i], acc[a][b + 1][i], limit, alpha));
+        }
+        continue;
+      }
 #pragma unroll
       for (int b = 0; b < 4; b++) {
         int n = n0 + wn + b * 16 + n16;
@@ -358,7 +389,7 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 expert_gemm_fma_k(const T* __restrict__ x, int ldx, int x_div, const T* __restrict__ w,
                   const int* __restrict__ cnt, const int* __restrict__ rows, int ldr,
-                  T* __restrict__ out, int ldo, int N, int K, int E, int TMP) {
+                  T* __restrict__ out, int ldo, int N, int K, int E, int TMP, int epi, float limit, float alpha) {
   __shared__ float sx[32][EG_KT + 1];
   __shared__ float sw[64][EG_KT + 1];
   __shared__ int sslot[32];
@@ -402,6 +433,15 @@ expert_gemm_fma_k(const T* __restrict__ x, int ldx, int x_div, const T* __restri
   for (int a = 0; a < 2; a++) {
     int s = sslot[ty * 2 + a];
     if (s < 0) continue;
+    if (epi) {
+#pragma unroll
+      for (int u = 0; u < 4; u += 2) {
+        int n = n0 + 16 * u;
+        if (n + 16 + tx < N)
+          stf(out, (size_t)s * ldo + n / 2 + tx, expert_act(acc[a][u], acc[a][u + 1], limit, alpha));
+      }
+      continue;
+    }
 #pragma unroll
     for (int u = 0; u < 4; u++) {
       int n = n0 + tx + 16 * u;
@@ -438,31 +478,34 @@ int p2p_sm_group_route(const void* h, int ldh, const float* wr, int R, int W, in
   return (int)hipGetLastError();
 }
 
-// total_slots: slots over all experts (rows * top; every slot is in exactly one list)
+// total_slots: slots over all experts (rows * top; every slot is in exactly one list).
+// epi = 1: w holds gate / up rows interleaved in groups of 16 (N = 2F rows, a multiple of 32)
+// and out [slots, F] receives the experts' activation instead of the raw products.
 int p2p_sm_expert_gemm(const void* x, int ldx, int x_div, const void* w, const int* cnt,
                        const int* rows, int ldr, void* out, int ldo, int E, int N, int K,
-                       int total_slots, int f32, hipStream_t st) {
+                       int total_slots, int epi, float limit, float alpha, int f32,
+                       hipStream_t st) {
   if (total_slots <= 0 || E <= 0) return 0;
-  if (x_div < 1 || N < 1 || K < 1) return (int)hipErrorInvalidValue;
+  if (x_div < 1 || N < 1 || K < 1 || (epi && N % 32)) return (int)hipErrorInvalidValue;
   if (!f32 && K % 8 == 0 && ldx % 8 == 0 && ((size_t)x & 15) == 0 && ((size_t)w & 15) == 0) {
     if (total_slots >= 64 * E) {   // prompts: the large tile
       int tmp = (((total_slots + 127) / 128 + E) + 7) & ~7;
       dim3 grid(tmp * ((N + 127) / 128));
       hipLaunchKernelGGL(expert_gemm_mfma_big_k, grid, dim3(256), 0, st, (const bf16*)x, ldx, x_div,
-                         (const bf16*)w, cnt, rows, ldr, (bf16*)out, ldo, N, K, E, tmp);
+                         (const bf16*)w, cnt, rows, ldr, (bf16*)out, ldo, N, K, E, tmp, epi, limit, alpha);
       return (int)hipGetLastError();
     }
     int tmp = (((total_slots + 15) / 16 + E) + 7) & ~7;
     dim3 grid(tmp * ((N + 63) / 64));
     hipLaunchKernelGGL(expert_gemm_mfma_k, grid, dim3(256), 0, st, (const bf16*)x, ldx, x_div,
-                       (const bf16*)w, cnt, rows, ldr, (bf16*)out, ldo, N, K, E, tmp);
+                       (const bf16*)w, cnt, rows, ldr, (bf16*)out, ldo, N, K, E, tmp, epi, limit, alpha);
     return (int)hipGetLastError();
   }
   int tmp = (((total_slots + 31) / 32 + E) + 7) & ~7;
   dim3 grid(tmp * ((N + 63) / 64));
   SM_DISPATCH_T(f32, hipLaunchKernelGGL(expert_gemm_fma_k<T>, grid, dim3(256), 0, st,
                                          (const T*)x, ldx, x_div, (const T*)w, cnt, rows, ldr,
-                                         (T*)out, ldo, N, K, E, tmp));
+                                         (T*)out, ldo, N, K, E, tmp, epi, limit, alpha));
   return (int)hipGetLastError();
 }
 

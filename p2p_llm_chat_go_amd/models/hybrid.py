@@ -644,8 +644,13 @@ class MoEFF:
 
     def load(self, get, dtype, dev):
         self.wr = get("router").to(dev).float().contiguous()
-        self.w_gu = torch.stack([torch.cat([get("e%d.gate" % e), get("e%d.up" % e)], 0)
-                                 for e in range(self.E)]).to(dev, dtype).contiguous()
+        gate = torch.stack([get("e%d.gate" % e) for e in range(self.E)])
+        up = torch.stack([get("e%d.up" % e) for e in range(self.E)])
+        # widths that are multiples of 16: gate and up rows interleaved, so that the first
+        # product's epilogue applies the activation (otherwise gate | up and a pointwise pass)
+        self.fused = self.F % 16 == 0
+        w_gu = sm.interleave_gate_up(gate, up) if self.fused else torch.cat([gate, up], 1)
+        self.w_gu = w_gu.to(dev, dtype).contiguous()
         self.w_down = torch.stack([get("e%d.down" % e) for e in range(self.E)]).to(dev, dtype).contiguous()
 
     def forward(self, h):
@@ -655,10 +660,13 @@ class MoEFF:
         cnt = torch.empty(self.E, device=dev, dtype=torch.int32)
         rows = torch.empty(self.E, R * top, device=dev, dtype=torch.int32)
         sm.group_route(h, self.wr, top, self.groups, self.keep, ids, wts, cnt, rows)
-        gu = torch.empty(R * top, 2 * self.F, device=dev, dtype=h.dtype)
-        sm.expert_gemm(h, top, self.w_gu, cnt, rows, gu, R * top)
         act = torch.empty(R * top, self.F, device=dev, dtype=h.dtype)
-        sm.ff_act(gu, act, self.limit)
+        if self.fused:
+            sm.expert_gemm(h, top, self.w_gu, cnt, rows, act, R * top, act_limit=self.limit)
+        else:
+            gu = torch.empty(R * top, 2 * self.F, device=dev, dtype=h.dtype)
+            sm.expert_gemm(h, top, self.w_gu, cnt, rows, gu, R * top)
+            sm.ff_act(gu, act, self.limit)
         y = torch.empty(R * top, self.width, device=dev, dtype=h.dtype)
         sm.expert_gemm(act, 1, self.w_down, cnt, rows, y, R * top)
         out = torch.empty(R, self.width, device=dev, dtype=h.dtype)

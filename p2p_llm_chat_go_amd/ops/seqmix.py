@@ -1,6 +1,8 @@
-"""Sequence-mixer ops: recurrent state layers (generalized delta rule, Mamba-2), latent
-attention with a sliding window and a softmax sink, learned positions, and the norms and
-pointwise steps around them.
+"""Sequence-mixer ops: recurrent state layers (generalized delta rule, Mamba-2, gated delta
+rule, HGRN2), latent attention and grouped-query attention with a sliding window and a
+softmax sink (query/key norm, rotary positions and the cache write in one pass), a
+group-limited expert router with grouped expert products, learned positions, and the norms
+and pointwise steps around them.
 
 GPU tensors always run the gfx950 kernels of ``csrc/seqmix`` (``libp2p_seqmix.so``, built on
 first use when missing); CPU tensors run the PyTorch rendering of the same math, which is
@@ -96,7 +98,8 @@ _SIGS = {
     "p2p_sm_group_route": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                            c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "p2p_sm_expert_gemm": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-                           c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                           c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
+                           c_void_p],
     "p2p_sm_expert_combine": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                               c_int, c_void_p],
 }
@@ -980,26 +983,53 @@ def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows):
     return ids, wts
 
 
-def expert_gemm(x, x_div: int, w, cnt, rows, out, total_slots: int):
+def interleave_gate_up(gate, up):
+    """[..., F, K] gate and up rows -> [..., 2F, K] as 16 gate rows, their 16 up rows, the next
+    16 gate rows, ... (F a multiple of 16): the layout ``expert_gemm`` wants for its fused
+    activation."""
+    F, K = gate.shape[-2:]
+    lead = gate.shape[:-2]
+    g = gate.reshape(*lead, F // 16, 1, 16, K)
+    u = up.reshape(*lead, F // 16, 1, 16, K)
+    return torch.cat([g, u], dim=-3).reshape(*lead, 2 * F, K)
+
+
+def expert_gemm(x, x_div: int, w, cnt, rows, out, total_slots: int, act_limit=None,
+                act_alpha: float = 1.702):
     """Per expert e and each of its routed slots s = rows[e, i] (i < cnt[e]):
     out[s] = x[s // x_div] @ w[e]^T.  w [E, N, K] (activation type), x [*, K], out [slots, N].
     total_slots: the slots over all experts (every slot is in exactly one list; the grid is
     sized from it, so no launch depends on the counts).  Accumulation is fp32; a slot's
-    result does not depend on the other slots."""
+    result does not depend on the other slots.
+    act_limit: w = ``interleave_gate_up(gate, up)`` and out [slots, N/2] receives
+    min(g, L) * sigmoid(alpha * min(g, L)) * (clamp(u, -L, L) + 1) of the two products (fp32
+    before the rounding) instead of the products themselves."""
     E, N, K = w.shape
+    fused = act_limit is not None
     if not x.is_cuda:
         for e in range(E):
             sl = rows[e, :int(cnt[e])].long()
-            if sl.numel():
-                out[sl] = torch.nn.functional.linear(x[sl // x_div], w[e])
+            if not sl.numel():
+                continue
+            y = torch.nn.functional.linear(x[sl // x_div].float(), w[e].float())
+            if fused:
+                y = y.view(-1, N // 32, 2, 16)
+                g = torch.clamp(y[:, :, 0], max=act_limit)
+                u = torch.clamp(y[:, :, 1], -act_limit, act_limit)
+                y = (g * torch.sigmoid(act_alpha * g) * (u + 1)).reshape(-1, N // 2)
+            out[sl] = y.to(out.dtype)
         return out
     _rows2d(x, "x")
     _rows2d(out, "out")
-    assert w.is_contiguous() and x.shape[1] == K and out.shape[1] == N
+    assert w.is_contiguous() and x.shape[1] == K and out.shape[1] == (N // 2 if fused else N)
     assert x.dtype == w.dtype == out.dtype and cnt.numel() == E
+    if fused and N % 32:
+        raise ValueError("fused expert activation needs gate / up widths that are multiples of 16")
     _chk(lib().p2p_sm_expert_gemm(x.data_ptr(), x.stride(0), x_div, w.data_ptr(), cnt.data_ptr(),
                                   rows.data_ptr(), rows.stride(0), out.data_ptr(), out.stride(0),
-                                  E, N, K, total_slots, _f32(x), _st(x)), "expert_gemm")
+                                  E, N, K, total_slots, 1 if fused else 0,
+                                  float(act_limit) if fused else 0.0, act_alpha, _f32(x), _st(x)),
+         "expert_gemm")
     return out
 
 

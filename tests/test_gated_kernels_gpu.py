@@ -186,7 +186,8 @@ def test_gated_delta_scan(dt, H, G, D, V, taps, lens):
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("E,groups,keep,top,W,Fd", [(12, 3, 2, 3, 72, 40), (8, 1, 1, 2, 64, 64),
-                                                     (6, 6, 2, 2, 50, 33), (70, 7, 3, 5, 96, 24)])
+                                                     (6, 6, 2, 2, 50, 33), (70, 7, 3, 5, 96, 24),
+                                                     (5, 1, 1, 3, 40, 48)])
 @pytest.mark.parametrize("R", [45, 300])     # few slots per expert / the large prompt tile
 def test_experts(dt, E, groups, keep, top, W, Fd, R):
     g = torch.Generator().manual_seed(5)
@@ -217,6 +218,14 @@ def test_experts(dt, E, groups, keep, top, W, Fd, R):
     sm.expert_gemm(h, top, wg, c1, r1, gu1, R * top)
     sm.expert_gemm(h.to(DEV), top, wg.to(DEV), c2.to(DEV), r2.to(DEV), gu2, R * top)
     torch.testing.assert_close(gu2.cpu().float(), gu1.float(), **_tol(dt))
+    if Fd % 16 == 0:    # the activation in the first product's epilogue
+        wi = sm.interleave_gate_up(wg[:, :Fd], wg[:, Fd:])
+        a0 = sm.ff_act(gu1, torch.empty(R * top, Fd, dtype=dt), 0.9)
+        a1 = sm.expert_gemm(h, top, wi, c1, r1, torch.zeros(R * top, Fd, dtype=dt), R * top, act_limit=0.9)
+        a2 = sm.expert_gemm(h.to(DEV), top, wi.to(DEV), c2.to(DEV), r2.to(DEV),
+                            torch.zeros(R * top, Fd, dtype=dt, device=DEV), R * top, act_limit=0.9)
+        torch.testing.assert_close(a1.float(), a0.float(), **_tol(dt))
+        torch.testing.assert_close(a2.cpu().float(), a1.float(), **_tol(dt))
     act = torch.randn(R * top, Fd, generator=g).to(dt)
     y1, y2 = torch.zeros(R * top, W, dtype=dt), torch.zeros(R * top, W, dtype=dt, device=DEV)
     sm.expert_gemm(act, 1, wd, c1, r1, y1, R * top)
